@@ -31,7 +31,8 @@ def plan_group_pages(groups, page_size: int, num_blocks: int, kv_cache_bytes, it
     """Pages of every cache group.  groups: the layout's CacheGroupSpec list (n_kv_head, head_dim,
     window, n_pools).  Without kv_cache_bytes every group gets num_blocks pages (the one-group
     shorthand, the reference's num_blocks).  With it the bytes are split so that every group holds
-    the same number of full-length requests: a group's page costs n_pools * 2 * n_kv_head * page_size
+    the same number of full-length requests: a group's page costs n_pools * 2 (1 where keys and values
+    are one joint tensor) * n_kv_head * page_size
     * head_dim * itemsize bytes, and a full-length request holds its whole span in a group that
     keeps all keys but only a window (and the page being written) in one that keeps a window."""
     if kv_cache_bytes is None:
@@ -39,7 +40,7 @@ def plan_group_pages(groups, page_size: int, num_blocks: int, kv_cache_bytes, it
     span_all = int(max_positions) if max_positions else NOMINAL_SPAN
     page_bytes, pages_per_request = [], []
     for g in groups:
-        page_bytes.append(g.n_pools * 2 * g.n_kv_head * page_size * g.head_dim * itemsize)
+        page_bytes.append(g.n_pools * (1 if getattr(g, "joint", False) else 2) * g.n_kv_head * page_size * g.head_dim * itemsize)
         span = min(g.window + page_size, span_all) if g.window else span_all
         pages_per_request.append(-(-span // page_size))
     per_request = sum(b * n for b, n in zip(page_bytes, pages_per_request))

@@ -1,0 +1,197 @@
+// Gated feed-forwards and experts chosen by a table.
+//
+// gated unit: act[n][j] = silu(z[n][j]) * z[n][F + j], z = the joint product with the gate and up
+// matrices stacked, silu(v) = v * sigmoid(v), in 32-bit.
+//
+// experts: a token's id picks a row of `top` experts from an integer table.  A (token, choice)
+// pair is one unit of work.  The route kernel sorts the pairs by expert into slots; every expert's
+// run of slots is padded to a multiple of EX_TILE, so a tile of slots belongs to one expert
+// (tile_expert[tile], -1 for a tile that no expert uses) and slot_token[slot] is the pair's token
+// row (-1 for padding), slot_pair[slot] the pair's own index n * top + k.  The grouped product
+// then multiplies each tile by its expert's matrix; rows come from, and go to, the places that the
+// two index arrays name.  Every output element is one chain over k in order, whatever its slot.
+#include "common.h"
+#include "launchers.h"
+
+#define EX_TILE 16
+#define EX_BK 64
+#define EX_MAX_EXPERTS 1024
+
+template <typename T, bool FAST>
+__global__ void gated_unit_kernel(const T* __restrict__ z, long ldz, T* __restrict__ act, long lda, long total,
+                                  int hidden) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long n = i / hidden;
+  const int j = (int)(i - n * hidden);
+  const float g = to_float<T>(z[n * ldz + j]), u = to_float<T>(z[n * ldz + hidden + j]);
+  const float s = FAST ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) : g / (1.0f + expf(-g));
+  act[n * lda + j] = from_float<T>(s * u);
+}
+
+extern "C" int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype,
+                               int fast, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!z || !act) return MGPT_ERR_NULL;
+  if (n_rows < 0 || hidden <= 0 || ldz < 2L * hidden || lda < hidden) return MGPT_ERR_BAD_SHAPE;
+  const long total = (long)n_rows * hidden;
+  const long blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((unsigned)blocks), block(256);
+#define GU_LAUNCH(T, F) \
+  hipLaunchKernelGGL((gated_unit_kernel<T, F>), grid, block, 0, stream, (const T*)z, ldz, (T*)act, lda, total, hidden)
+  if (dtype == MGPT_F32) {
+    if (fast) GU_LAUNCH(float, true); else GU_LAUNCH(float, false);
+  } else if (dtype == MGPT_BF16) {
+    if (fast) GU_LAUNCH(bf16_t, true); else GU_LAUNCH(bf16_t, false);
+  } else {
+    return MGPT_ERR_BAD_DTYPE;
+  }
+#undef GU_LAUNCH
+  return mgpt_last_error();
+}
+
+// One workgroup: counts the pairs of every expert, lays the experts' runs of slots out one after
+// the other (each padded to whole tiles), and deals the pairs into them.
+__global__ __launch_bounds__(256) void expert_route_kernel(
+    const int* __restrict__ ids, const int* __restrict__ q_req, const int* __restrict__ table, int top,
+    int n_rows, int n_experts, int* __restrict__ slot_token, int* __restrict__ slot_pair,
+    int* __restrict__ tile_expert, int n_slots, int n_tiles) {
+  __shared__ int count[EX_MAX_EXPERTS];
+  __shared__ int start[EX_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < n_experts; e += blockDim.x) count[e] = 0;
+  for (int s = tid; s < n_slots; s += blockDim.x) slot_token[s] = -1;
+  for (int t = tid; t < n_tiles; t += blockDim.x) tile_expert[t] = -1;
+  __syncthreads();
+  const int n_pairs = n_rows * top;
+  for (int p = tid; p < n_pairs; p += blockDim.x) {
+    const int n = p / top;
+    if (q_req && q_req[n] < 0) continue;   // padded token
+    const int e = table[(long)ids[n] * top + (p - n * top)];
+    if (e >= 0 && e < n_experts) atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < n_experts; ++e) {
+      start[e] = at;
+      const int tiles = (count[e] + EX_TILE - 1) / EX_TILE;
+      for (int t = 0; t < tiles; ++t) tile_expert[at / EX_TILE + t] = e;
+      at += tiles * EX_TILE;
+      count[e] = 0;
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < n_pairs; p += blockDim.x) {
+    const int n = p / top;
+    if (q_req && q_req[n] < 0) continue;
+    const int e = table[(long)ids[n] * top + (p - n * top)];
+    if (e < 0 || e >= n_experts) continue;
+    const int s = start[e] + atomicAdd(&count[e], 1);
+    slot_token[s] = n;
+    slot_pair[s] = p;
+  }
+}
+
+// n_slots >= n_rows * top + n_experts * (EX_TILE - 1) rounded up to whole tiles; n_tiles = n_slots / EX_TILE
+extern "C" int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows,
+                                 int n_experts, int* slot_token, int* slot_pair, int* tile_expert, int n_slots,
+                                 int n_tiles, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!ids || !table || !slot_token || !slot_pair || !tile_expert) return MGPT_ERR_NULL;
+  if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || n_slots != n_tiles * EX_TILE)
+    return MGPT_ERR_BAD_SHAPE;
+  // every expert that is used wastes less than a tile
+  const long pairs = (long)n_rows * top;
+  const long worst = pairs + (n_experts < pairs ? n_experts : pairs) * (long)(EX_TILE - 1);
+  if ((long)n_slots < worst / EX_TILE * EX_TILE) return MGPT_ERR_BAD_SHAPE;
+  hipLaunchKernelGGL(expert_route_kernel, dim3(1), dim3(256), 0, stream, ids, q_req, table, top, n_rows, n_experts,
+                     slot_token, slot_pair, tile_expert, n_slots, n_tiles);
+  return mgpt_last_error();
+}
+
+template <typename T, typename OT>
+__global__ __launch_bounds__(256) void grouped_linear_kernel(
+    const T* __restrict__ A, long lda, const int* __restrict__ a_rows, const T* __restrict__ W, long w_stride,
+    const int* __restrict__ tile_expert, const int* __restrict__ slot_token, OT* __restrict__ out, long ldo,
+    const int* __restrict__ out_rows, int n_out, int k_dim) {
+  __shared__ float As[EX_TILE][EX_BK + 1];
+  __shared__ float Ws[EX_TILE][EX_BK + 1];
+  const int tile = blockIdx.y;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int tid = threadIdx.x;
+  const int r = tid >> 4, c = tid & 15;
+  const int sk = (tid & 15) * 4;
+  const int col0 = blockIdx.x * EX_TILE;
+  const int slot = tile * EX_TILE + r;
+  const bool a_ok = slot_token[slot] >= 0, w_ok = col0 + r < n_out;
+  const long arow = a_ok ? (a_rows ? a_rows[slot] : slot) : 0;
+  const T* ap = A + arow * lda + sk;
+  const T* wp = W + (long)e * w_stride + (long)(col0 + r) * k_dim + sk;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < k_dim; k0 += EX_BK) {
+    const int kmax = k_dim - k0 < EX_BK ? k_dim - k0 : EX_BK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool k_ok = sk + i < kmax;
+      As[r][sk + i] = (a_ok && k_ok) ? to_float<T>(ap[k0 + i]) : 0.f;
+      Ws[r][sk + i] = (w_ok && k_ok) ? to_float<T>(wp[k0 + i]) : 0.f;
+    }
+    __syncthreads();
+    for (int kk = 0; kk < kmax; ++kk) acc = fmaf(As[r][kk], Ws[c][kk], acc);
+    __syncthreads();
+  }
+  const int col = col0 + c;
+  if (!a_ok || col >= n_out) return;
+  const long orow = out_rows ? out_rows[slot] : slot;
+  out[orow * ldo + col] = from_float<OT>(acc);
+}
+
+// out[out_rows[s] or s] = A[a_rows[s] or s] @ W[tile_expert[s / EX_TILE]]^T for every slot s with
+// slot_token[s] >= 0.  W: [experts][n_out][k_dim], w_stride elements from one expert to the next.
+extern "C" int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride,
+                                   const int* tile_expert, const int* slot_token, void* out, int out_dtype,
+                                   long ldo, const int* out_rows, int n_tiles, int n_out, int k_dim, int dtype,
+                                   hipStream_t stream) {
+  if (n_tiles == 0 || n_out == 0) return MGPT_OK;
+  if (!a || !w || !tile_expert || !slot_token || !out) return MGPT_ERR_NULL;
+  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out) return MGPT_ERR_BAD_SHAPE;
+  if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((n_out + EX_TILE - 1) / EX_TILE, n_tiles), block(256);
+#define GL_LAUNCH(T, OT)                                                                                     \
+  hipLaunchKernelGGL((grouped_linear_kernel<T, OT>), grid, block, 0, stream, (const T*)a, lda, a_rows,       \
+                     (const T*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows, n_out, k_dim)
+  if (dtype == MGPT_F32 && out_dtype == MGPT_F32) GL_LAUNCH(float, float);
+  else if (dtype == MGPT_BF16 && out_dtype == MGPT_BF16) GL_LAUNCH(bf16_t, bf16_t);
+  else if (dtype == MGPT_BF16 && out_dtype == MGPT_F32) GL_LAUNCH(bf16_t, float);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef GL_LAUNCH
+  return mgpt_last_error();
+}
+
+__global__ void expert_combine_kernel(const float* __restrict__ pair_out, float* __restrict__ y, long total,
+                                      int width, int top, float weight) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long n = i / width;
+  const int c = (int)(i - n * width);
+  float acc = 0.f;
+  for (int k = 0; k < top; ++k) acc += pair_out[(n * top + k) * (long)width + c];
+  y[i] += acc * weight;
+}
+
+// y[n] += weight * sum_k pair_out[n * top + k]
+extern "C" int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, int top, float weight,
+                                   hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!pair_out || !y) return MGPT_ERR_NULL;
+  if (n_rows < 0 || width <= 0 || top <= 0) return MGPT_ERR_BAD_SHAPE;
+  const long total = (long)n_rows * width;
+  const long blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(expert_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, pair_out, y, total, width,
+                     top, weight);
+  return mgpt_last_error();
+}

@@ -1,0 +1,115 @@
+// Latent attention's own steps: the RMS-normed latent stored into its pages, and the products
+// that every head makes with a matrix of its own (queries folded onto the latent basis before
+// attention, the attended latents unfolded into the head's values after it).
+//
+// A latent pool is [pages][1][page_size][rank]: one row per cached token, keys and values both
+// come from it, so slot s lies at s * rank.
+#include "common.h"
+#include "launchers.h"
+
+// c = v / sqrt(mean(v^2) + eps) * gain, statistics and product in 32-bit; one wave per token
+template <typename T>
+__global__ void rms_norm_store_kernel(const T* __restrict__ src, long ld, const float* __restrict__ gain,
+                                      float eps, T* __restrict__ pool, const int* __restrict__ slot_mapping,
+                                      int n_tokens, int rank) {
+  const int lane = threadIdx.x & (MGPT_WAVE - 1);
+  const int row = blockIdx.x * (blockDim.x / MGPT_WAVE) + (threadIdx.x / MGPT_WAVE);
+  if (row >= n_tokens) return;
+  const int slot = slot_mapping[row];
+  if (slot < 0) return;  // padded row
+  const T* r = src + (long)row * ld;
+  float ss = 0.f;
+  for (int c = lane; c < rank; c += MGPT_WAVE) {
+    const float v = to_float<T>(r[c]);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)rank + eps);
+  T* dst = pool + (long)slot * rank;
+  for (int c = lane; c < rank; c += MGPT_WAVE) dst[c] = from_float<T>(to_float<T>(r[c]) * inv * gain[c]);
+}
+
+// src: [n_tokens, rank] with row stride ld (already offset to the latent's columns); pool: the
+// latent pages, same dtype.
+extern "C" int mgpt_rms_norm_store(const void* src, int dtype, long ld, const float* gain, float eps, void* pool,
+                                   const int* slot_mapping, int n_tokens, int rank, hipStream_t stream) {
+  if (n_tokens == 0) return MGPT_OK;
+  if (!src || !gain || !pool || !slot_mapping) return MGPT_ERR_NULL;
+  if (n_tokens < 0 || rank <= 0 || ld < rank) return MGPT_ERR_BAD_SHAPE;
+  dim3 grid((n_tokens + 3) / 4), block(4 * MGPT_WAVE);
+  if (dtype == MGPT_F32)
+    hipLaunchKernelGGL(rms_norm_store_kernel<float>, grid, block, 0, stream, (const float*)src, ld, gain, eps,
+                       (float*)pool, slot_mapping, n_tokens, rank);
+  else if (dtype == MGPT_BF16)
+    hipLaunchKernelGGL(rms_norm_store_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, ld, gain, eps,
+                       (bf16_t*)pool, slot_mapping, n_tokens, rank);
+  else
+    return MGPT_ERR_BAD_DTYPE;
+  return mgpt_last_error();
+}
+
+// out[n][h][o] = sum_i a[n][h][i] * w[h][o][i], optionally times sigmoid(gate[n][h][o]).
+// A workgroup owns 16 rows x 16 columns of one head, one element a thread; k runs 0..K-1 in order
+// for every element, so a row's result does not depend on the other rows of the launch.
+#define HL_TILE 16
+#define HL_BK 64
+
+template <typename T, bool FAST>
+__global__ __launch_bounds__(256) void heads_linear_kernel(
+    const T* __restrict__ A, long lda, const T* __restrict__ W, T* __restrict__ out, long ldo,
+    const T* __restrict__ gate, long ldg, int n_rows, int n_out, int k_dim) {
+  __shared__ float As[HL_TILE][HL_BK + 1];
+  __shared__ float Ws[HL_TILE][HL_BK + 1];
+  const int tid = threadIdx.x, head = blockIdx.z;
+  const int r = tid >> 4, c = tid & 15;
+  const int sk = (tid & 15) * 4;
+  const int row0 = blockIdx.y * HL_TILE, col0 = blockIdx.x * HL_TILE;
+  const bool a_ok = row0 + r < n_rows, w_ok = col0 + r < n_out;
+  const T* ap = A + (long)(row0 + r) * lda + (long)head * k_dim + sk;
+  const T* wp = W + ((long)head * n_out + col0 + r) * (long)k_dim + sk;
+  float acc = 0.f;
+  for (int k0 = 0; k0 < k_dim; k0 += HL_BK) {
+    const int kmax = k_dim - k0 < HL_BK ? k_dim - k0 : HL_BK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool k_ok = sk + i < kmax;
+      As[r][sk + i] = (a_ok && k_ok) ? to_float<T>(ap[k0 + i]) : 0.f;
+      Ws[r][sk + i] = (w_ok && k_ok) ? to_float<T>(wp[k0 + i]) : 0.f;
+    }
+    __syncthreads();
+    for (int kk = 0; kk < kmax; ++kk) acc = fmaf(As[r][kk], Ws[c][kk], acc);
+    __syncthreads();
+  }
+  const int row = row0 + r, col = col0 + c;
+  if (row >= n_rows || col >= n_out) return;
+  float v = acc;
+  if (gate) {
+    const float g = to_float<T>(gate[(long)row * ldg + (long)head * n_out + col]);
+    v *= FAST ? __builtin_amdgcn_rcpf(1.0f + __expf(-g)) : 1.0f / (1.0f + expf(-g));
+  }
+  out[(long)row * ldo + (long)head * n_out + col] = from_float<T>(v);
+}
+
+extern "C" int mgpt_heads_linear(const void* a, long lda, const void* w, void* out, long ldo, const void* gate,
+                                 long ldg, int n_rows, int n_head, int n_out, int k_dim, int dtype, int fast,
+                                 hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!a || !w || !out) return MGPT_ERR_NULL;
+  if (n_rows < 0 || n_head <= 0 || n_out <= 0 || k_dim <= 0 || lda < (long)n_head * k_dim ||
+      ldo < (long)n_head * n_out || (gate && ldg < (long)n_head * n_out))
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_head > 65535 || (n_rows + HL_TILE - 1) / HL_TILE > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((n_out + HL_TILE - 1) / HL_TILE, (n_rows + HL_TILE - 1) / HL_TILE, n_head), block(256);
+#define HL_LAUNCH(T, F)                                                                                   \
+  hipLaunchKernelGGL((heads_linear_kernel<T, F>), grid, block, 0, stream, (const T*)a, lda, (const T*)w,  \
+                     (T*)out, ldo, (const T*)gate, ldg, n_rows, n_out, k_dim)
+  if (dtype == MGPT_F32) {
+    if (fast) HL_LAUNCH(float, true); else HL_LAUNCH(float, false);
+  } else if (dtype == MGPT_BF16) {
+    if (fast) HL_LAUNCH(bf16_t, true); else HL_LAUNCH(bf16_t, false);
+  } else {
+    return MGPT_ERR_BAD_DTYPE;
+  }
+#undef HL_LAUNCH
+  return mgpt_last_error();
+}

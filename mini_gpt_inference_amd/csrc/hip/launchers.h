@@ -28,7 +28,7 @@ int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, voi
 int mgpt_paged_attention_generic(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int dtype,
-    int fast_exp, hipStream_t stream);
+    int fast_exp, const float* sinks, hipStream_t stream);
 // attention_prefill.hip
 int mgpt_prefill_attention_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req, int
@@ -110,6 +110,30 @@ int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int
     slot_mapping, const int* block_tables, const int* page_sizes, int n_groups, int n_stride, int r_stride,
     int max_blocks, int* history, int* history_pos, int history_rows, int history_stride, const float*
     tile_best, const int* tile_best_idx, int n_tiles, hipStream_t stream);
+// streams.hip
+int mgpt_embed_scaled(const int* ids, const void* tok, float* x, int n_tokens, int width, int table_dtype, float
+    scale, int copies, hipStream_t stream);
+int mgpt_streams_read(const float* x, const float* coef, float* u, float* zero, int n_rows, int width, int
+    streams, hipStream_t stream);
+int mgpt_streams_write(float* x, const float* mix, const float* out, const float* y, int n_rows, int width, int
+    streams, hipStream_t stream);
+int mgpt_scale_softcap(float* logits, long ld, int n_rows, int vocab, float scale, float cap, int fast,
+    hipStream_t stream);
+// latent.hip
+int mgpt_rms_norm_store(const void* src, int dtype, long ld, const float* gain, float eps, void* pool, const int*
+    slot_mapping, int n_tokens, int rank, hipStream_t stream);
+int mgpt_heads_linear(const void* a, long lda, const void* w, void* out, long ldo, const void* gate, long ldg,
+    int n_rows, int n_head, int n_out, int k_dim, int dtype, int fast, hipStream_t stream);
+// experts.hip
+int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype, int fast,
+    hipStream_t stream);
+int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows, int n_experts,
+    int* slot_token, int* slot_pair, int* tile_expert, int n_slots, int n_tiles, hipStream_t stream);
+int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
+    tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
+    int n_out, int k_dim, int dtype, hipStream_t stream);
+int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, int top, float weight,
+    hipStream_t stream);
 }
 
 // MGPT_FOR_EACH_LAUNCHER(X) expands X(name) for every launcher above
@@ -137,4 +161,14 @@ int mgpt_sample_advance(const float* logits, long ld, int n_rows, int vocab, int
   X(mgpt_linear_head_best) \
   X(mgpt_linear_decode_parts) \
   X(mgpt_sample) \
-  X(mgpt_sample_advance)
+  X(mgpt_sample_advance) \
+  X(mgpt_embed_scaled) \
+  X(mgpt_streams_read) \
+  X(mgpt_streams_write) \
+  X(mgpt_scale_softcap) \
+  X(mgpt_rms_norm_store) \
+  X(mgpt_heads_linear) \
+  X(mgpt_gated_unit) \
+  X(mgpt_expert_route) \
+  X(mgpt_grouped_linear) \
+  X(mgpt_expert_combine)

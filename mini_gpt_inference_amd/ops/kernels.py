@@ -97,6 +97,11 @@ def _need_i32(name: str, t: torch.Tensor, n: int) -> None:
           f"{name} must be a contiguous int32 buffer of at least {n} entries")
 
 
+def _need_sinks(sinks: Optional[torch.Tensor], n_head: int) -> None:
+    _need(sinks is None or (sinks.is_cuda and sinks.dtype == torch.float32 and sinks.is_contiguous()
+                            and sinks.numel() == n_head), "sinks must be float32 [n_head] on the GPU")
+
+
 def embed(ids: torch.Tensor, positions: Optional[torch.Tensor], table: torch.Tensor,
           pos_table: Optional[torch.Tensor], x: torch.Tensor, n_tokens: int) -> None:
     """x[t] = table[ids[t]] (+ pos_table[positions[t]]), into the float32 residual stream."""
@@ -195,15 +200,17 @@ def _check_attention_args(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, 
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                             block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                             q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
-                            window: int = 0, fast_exp: bool = False) -> None:
-    """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype)."""
+                            window: int = 0, fast_exp: bool = False, sinks: Optional[torch.Tensor] = None) -> None:
+    """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype).
+    sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h."""
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
     _need(head_dim <= 256, f"head size {head_dim} exceeds the kernel's limit of 256")
+    _need_sinks(sinks, n_head)
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _stream())
+        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), _stream())
     _check(rc, "paged_attention_generic")
 
 
@@ -916,3 +923,188 @@ def residual_settle(pending, settled: torch.Tensor, n_rows: int) -> bool:
         return False
     _check(rc, "residual_settle")
     return True
+
+
+# ---------------------------------------------------------------- several residual streams, soft-capped logits
+MAX_STREAMS = 8
+
+
+def embed_scaled(ids: torch.Tensor, table: torch.Tensor, x: torch.Tensor, n_tokens: int, scale: float,
+                 copies: int = 1) -> None:
+    """x[t][s] = table[ids[t]] * scale for every s < copies; x is float32 [>=n_tokens, copies * width]."""
+    _need_cuda(ids, table, x)
+    width = table.shape[1]
+    _need(table.dim() == 2 and table.is_contiguous(), "embedding table must be dense [vocab, width]")
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[1] == copies * width and x.shape[0] >= n_tokens,
+          "residual streams must be dense float32 [>=n_tokens, copies * width]")
+    _need_i32("ids", ids, n_tokens)
+    rc = library.kernels().mgpt_embed_scaled(_ptr(ids), _ptr(table), _ptr(x), n_tokens, width, _dtype_code(table),
+                                             float(scale), int(copies), _stream())
+    _check(rc, "embed_scaled")
+
+
+def _need_streams(x: torch.Tensor, n_rows: int, width: int, streams: int) -> None:
+    _need(1 <= streams <= MAX_STREAMS, f"the kernels take up to {MAX_STREAMS} residual streams")
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2 and x.shape[1] == streams * width
+          and x.shape[0] >= n_rows, "residual streams must be dense float32 [>=n_rows, streams * width]")
+
+
+def _need_rows_f32(name: str, t: torch.Tensor, n_rows: int, width: int) -> None:
+    _need(t.dtype == torch.float32 and t.is_contiguous() and t.dim() == 2 and t.shape[1] == width
+          and t.shape[0] >= n_rows, f"{name} must be dense float32 [>=n_rows, {width}]")
+
+
+def streams_read(x: torch.Tensor, coef: Optional[torch.Tensor], u: torch.Tensor, n_rows: int, streams: int,
+                 zero: Optional[torch.Tensor] = None) -> None:
+    """u[n] = sum_s coef[s] x[n][s] (coef None: the plain sum); `zero`, shaped like u, is cleared."""
+    _need_cuda(x, coef, u, zero)
+    width = u.shape[1]
+    _need_streams(x, n_rows, width, streams)
+    _need_rows_f32("u", u, n_rows, width)
+    if zero is not None:
+        _need_rows_f32("zero", zero, n_rows, width)
+    _need(coef is None or (coef.dtype == torch.float32 and coef.is_contiguous() and coef.numel() == streams),
+          "coef must be float32 [streams]")
+    rc = library.kernels().mgpt_streams_read(_ptr(x), _ptr(coef), _ptr(u), _ptr(zero), n_rows, width, streams,
+                                             _stream())
+    _check(rc, "streams_read")
+
+
+def streams_write(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, y: torch.Tensor, n_rows: int,
+                  streams: int) -> None:
+    """x[n][t] = sum_s mix[s][t] x[n][s] + out[t] y[n], every t from the old streams."""
+    _need_cuda(x, mix, out, y)
+    width = y.shape[1]
+    _need_streams(x, n_rows, width, streams)
+    _need_rows_f32("y", y, n_rows, width)
+    _need(mix.dtype == torch.float32 and mix.is_contiguous() and tuple(mix.shape) == (streams, streams),
+          "mix must be float32 [streams, streams]")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and out.numel() == streams, "out must be float32 [streams]")
+    rc = library.kernels().mgpt_streams_write(_ptr(x), _ptr(mix), _ptr(out), _ptr(y), n_rows, width, streams,
+                                              _stream())
+    _check(rc, "streams_write")
+
+
+def scale_softcap(logits: torch.Tensor, n_rows: int, scale: float, cap: float, fast: bool) -> None:
+    """logits = cap * tanh(logits * scale / cap) in place (cap <= 0: the scale alone)."""
+    _need_cuda(logits)
+    _need(logits.dtype == torch.float32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.shape[0] >= n_rows,
+          "logits must be float32 [>=n_rows, vocab] with unit inner stride")
+    rc = library.kernels().mgpt_scale_softcap(_ptr(logits), logits.stride(0), n_rows, logits.shape[1], float(scale),
+                                              float(cap), int(fast), _stream())
+    _check(rc, "scale_softcap")
+
+
+# ---------------------------------------------------------------- latent attention
+def rms_norm_store(src: torch.Tensor, gain: torch.Tensor, eps: float, pool: torch.Tensor,
+                   slot_mapping: torch.Tensor, n_tokens: int) -> None:
+    """pool[slot of token n] = src[n] / sqrt(mean(src[n]^2) + eps) * gain; pool [pages, 1, page_size, rank]."""
+    _need_cuda(src, gain, pool, slot_mapping)
+    _need(pool.dim() == 4 and pool.shape[1] == 1 and pool.is_contiguous(),
+          "a latent pool must be dense [pages, 1, page_size, rank]")
+    rank = pool.shape[3]
+    _need(src.dim() == 2 and src.stride(1) == 1 and src.shape[1] == rank and src.shape[0] >= n_tokens
+          and src.dtype == pool.dtype, "latents must be [>=n_tokens, rank] in the pool's dtype")
+    _need(gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() == rank, "gain must be float32 [rank]")
+    _need_i32("slot_mapping", slot_mapping, n_tokens)
+    rc = library.kernels().mgpt_rms_norm_store(_ptr(src), _dtype_code(src), src.stride(0), _ptr(gain), float(eps),
+                                               _ptr(pool), _ptr(slot_mapping), n_tokens, rank, _stream())
+    _check(rc, "rms_norm_store")
+
+
+def heads_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_rows: int,
+                 gate: Optional[torch.Tensor] = None, fast: bool = False) -> None:
+    """out[n][h] = a[n][h] @ w[h].T for every head h, optionally times sigmoid(gate[n][h]).
+    w: [heads, n_out, k_dim]; a: [>=n_rows, >=heads * k_dim]; out, gate: [>=n_rows, >=heads * n_out]."""
+    _need_cuda(a, w, out, gate)
+    _need(w.dim() == 3 and w.is_contiguous(), "the heads' matrices must be dense [heads, out, in]")
+    n_head, n_out, k_dim = w.shape
+    _need(a.dtype == w.dtype == out.dtype and (gate is None or gate.dtype == a.dtype), "operands must share a dtype")
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] >= n_head * k_dim and a.shape[0] >= n_rows,
+          "activations must be [>=n_rows, >=heads * in] with unit inner stride")
+    for name, t in (("out", out), ("gate", gate)):
+        _need(t is None or (t.dim() == 2 and t.stride(1) == 1 and t.shape[1] >= n_head * n_out and t.shape[0] >= n_rows),
+              f"{name} must be [>=n_rows, >=heads * out] with unit inner stride")
+    rc = library.kernels().mgpt_heads_linear(_ptr(a), a.stride(0), _ptr(w), _ptr(out), out.stride(0), _ptr(gate),
+                                             0 if gate is None else gate.stride(0), n_rows, n_head, n_out, k_dim,
+                                             _dtype_code(a), int(fast), _stream())
+    _check(rc, "heads_linear")
+
+
+# ---------------------------------------------------------------- gated feed-forwards and experts
+EXPERT_TILE = 16
+MAX_EXPERTS = 1024
+
+
+def gated_unit(z: torch.Tensor, act: torch.Tensor, n_rows: int, hidden: int, fast: bool = False) -> None:
+    """act[n][j] = silu(z[n][j]) * z[n][hidden + j]."""
+    _need_cuda(z, act)
+    _need(z.dtype == act.dtype and z.dim() == 2 and act.dim() == 2 and z.stride(1) == 1 and act.stride(1) == 1
+          and z.shape[1] >= 2 * hidden and act.shape[1] >= hidden and z.shape[0] >= n_rows and act.shape[0] >= n_rows,
+          "z must be [>=n_rows, >=2 * hidden] and act [>=n_rows, >=hidden], one dtype")
+    rc = library.kernels().mgpt_gated_unit(_ptr(z), z.stride(0), _ptr(act), act.stride(0), n_rows, hidden,
+                                           _dtype_code(z), int(fast), _stream())
+    _check(rc, "gated_unit")
+
+
+def expert_slots(n_rows: int, top: int, n_experts: int) -> int:
+    """Slots that n_rows tokens with `top` experts each may need once every expert's run of slots is
+    padded to whole tiles."""
+    pairs = n_rows * top
+    worst = pairs + min(n_experts, pairs) * (EXPERT_TILE - 1)
+    return -(-worst // EXPERT_TILE) * EXPERT_TILE
+
+
+def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.Tensor, n_rows: int, n_experts: int,
+                 slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor) -> None:
+    """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip."""
+    _need_cuda(ids, q_req, table, slot_token, slot_pair, tile_expert)
+    _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "the table must be dense int32")
+    top = table.shape[1]
+    n_slots = expert_slots(n_rows, top, n_experts)
+    _need(n_experts <= MAX_EXPERTS, f"the route kernel takes up to {MAX_EXPERTS} experts")
+    _need_i32("ids", ids, n_rows)
+    if q_req is not None:
+        _need_i32("q_req", q_req, n_rows)
+    _need_i32("slot_token", slot_token, n_slots)
+    _need_i32("slot_pair", slot_pair, n_slots)
+    _need_i32("tile_expert", tile_expert, n_slots // EXPERT_TILE)
+    rc = library.kernels().mgpt_expert_route(_ptr(ids), _ptr(q_req), _ptr(table), top, n_rows, n_experts,
+                                             _ptr(slot_token), _ptr(slot_pair), _ptr(tile_expert), n_slots,
+                                             n_slots // EXPERT_TILE, _stream())
+    _check(rc, "expert_route")
+
+
+def grouped_linear(a: torch.Tensor, a_rows: Optional[torch.Tensor], w: torch.Tensor, tile_expert: torch.Tensor,
+                   slot_token: torch.Tensor, out: torch.Tensor, out_rows: Optional[torch.Tensor], n_slots: int) -> None:
+    """out[out_rows[s] or s] = a[a_rows[s] or s] @ w[expert of s's tile].T for every used slot s < n_slots.
+    w: [experts, n_out, k_dim]."""
+    _need_cuda(a, a_rows, w, tile_expert, slot_token, out, out_rows)
+    _need(w.dim() == 3 and w.is_contiguous(), "the experts' matrices must be dense [experts, out, in]")
+    _, n_out, k_dim = w.shape
+    _need(n_slots % EXPERT_TILE == 0, "slots come in whole tiles")
+    _need(a.dtype == w.dtype and a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim,
+          "activations must be [rows, in] in the matrices' dtype")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_out, "out must be [rows, out]")
+    _need(a_rows is not None or a.shape[0] >= n_slots, "activations have fewer rows than slots")
+    _need(out_rows is not None or out.shape[0] >= n_slots, "out has fewer rows than slots")
+    _need_i32("slot_token", slot_token, n_slots)
+    _need_i32("tile_expert", tile_expert, n_slots // EXPERT_TILE)
+    for t in (a_rows, out_rows):
+        if t is not None:
+            _need_i32("row index", t, n_slots)
+    rc = library.kernels().mgpt_grouped_linear(_ptr(a), a.stride(0), _ptr(a_rows), _ptr(w), w.stride(0),
+                                               _ptr(tile_expert), _ptr(slot_token), _ptr(out), _dtype_code(out),
+                                               out.stride(0), _ptr(out_rows), n_slots // EXPERT_TILE, n_out, k_dim,
+                                               _dtype_code(a), _stream())
+    _check(rc, "grouped_linear")
+
+
+def expert_combine(pair_out: torch.Tensor, y: torch.Tensor, n_rows: int, top: int, weight: float) -> None:
+    """y[n] += weight * sum_k pair_out[n * top + k]; both float32."""
+    _need_cuda(pair_out, y)
+    width = y.shape[1]
+    _need_rows_f32("y", y, n_rows, width)
+    _need_rows_f32("pair_out", pair_out, n_rows * top, width)
+    rc = library.kernels().mgpt_expert_combine(_ptr(pair_out), _ptr(y), n_rows, width, top, float(weight), _stream())
+    _check(rc, "expert_combine")

@@ -39,7 +39,7 @@ def kernels() -> ctypes.CDLL:
         lib.mgpt_layernorm.argtypes = [P, P, P, P, P, I, I, F, I, P]
         lib.mgpt_linear_generic.argtypes = [P, I, L, P, I, P, P, I, L, I, I, I, I, P]
         lib.mgpt_kv_write.argtypes = [P, I, L, I, I, P, P, P, I, I, I, I, P]
-        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P]
+        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P]
         lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P, P, I, P]
         lib.mgpt_sample_advance.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P,
                                             P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P, P, I, P]
@@ -147,6 +147,19 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_decode_parts_count": [],
         "mgpt_residual_settle": [P, P, I, L, P, P, P, P, P, I, I, P],
         "mgpt_fused_parts_limit": [I],
+        # several residual streams, scaled embedding, soft-capped logits
+        "mgpt_embed_scaled": [P, P, P, I, I, I, F, I, P],
+        "mgpt_streams_read": [P, P, P, P, I, I, I, P],
+        "mgpt_streams_write": [P, P, P, P, I, I, I, P],
+        "mgpt_scale_softcap": [P, L, I, I, F, F, I, P],
+        # latent attention
+        "mgpt_rms_norm_store": [P, I, L, P, F, P, P, I, I, P],
+        "mgpt_heads_linear": [P, L, P, P, L, P, L, I, I, I, I, I, I, P],
+        # gated feed-forwards and experts
+        "mgpt_gated_unit": [P, L, P, L, I, I, I, I, P],
+        "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, I, I, P],
+        "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, P],
+        "mgpt_expert_combine": [P, P, I, I, I, F, P],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name, None)

@@ -39,6 +39,7 @@ class KVNeed:
     n_kv_head: int
     head_dim: int
     window: int = 0   # 0: all earlier keys; w: the last w positions
+    joint: bool = False   # keys and values are one tensor (a latent that both are made from): a page holds it once
 
 
 @dataclass(frozen=True)
@@ -69,10 +70,13 @@ class Part:
         """Parameter name -> shape and role of every tensor this part needs."""
         return {}
 
-    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        """Receives the device tensors named by weight_requests (absent optional ones are missing)."""
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> Optional[Dict[str, torch.Tensor]]:
+        """Receives the device tensors named by weight_requests (absent optional ones are missing).
+        A part that joins some of them into one tensor may return parameter name -> the view of the
+        joint tensor that stands for it from now on; the model then lets go of the loaded one."""
         for name, tensor in tensors.items():
             setattr(self, name, tensor)
+        return None
 
 
 class Registry:

@@ -2,13 +2,13 @@
 
 from __future__ import annotations
 
-from typing import Mapping, Optional, Tuple
+from typing import Dict, Mapping, Optional, Tuple
 
 import torch
 
-from ..ops import residual
+from ..ops import kernels, residual
 from ..ops.linear import LazyNorm
-from .base import CacheBinding, Part, StepContext, register_arrangement
+from .base import CacheBinding, Part, StepContext, VECTOR, WeightRequest, register_arrangement
 from .feedforward import FeedForward
 from .mixers import Mixer
 from .positions import PositionEncoding
@@ -53,3 +53,50 @@ class PreNorm(Arrangement):
         if not feed_forward.takes_pending_residual:
             residual.settle(ctx, x, n)
         feed_forward.forward_add(ctx, LazyNorm(norm2, x, n), x)
+
+
+@register_arrangement("hyper_connections")
+class HyperConnections(Arrangement):
+    """A pre-norm layer over several residual streams.  A token's residual is S rows x_1 .. x_S.
+    For sublayer q (1: the mixer, 2: the feed-forward, which a layer may lack) with its own
+    a_q [S], M_q [S, S] and b_q [S]:
+
+        u = sum_s a_q[s] x_s;  y = sublayer_q(norm_q(u));  x_t <- sum_s M_q[s, t] x_s + b_q[t] y
+
+    every new stream from the old ones, all in float32.  With S = 1, a = b = 1 and M = 1 this is
+    the plain pre-norm layer.  The sublayers are the framework's ordinary parts: they add their
+    output into a cleared buffer that stands for y."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, streams: int, feed_forward: bool = True) -> None:
+        self.width, self.streams = int(width), int(streams)
+        if not 1 <= self.streams <= kernels.MAX_STREAMS:
+            raise ValueError(f"{self.streams} residual streams: the kernels take 1 to {kernels.MAX_STREAMS}")
+        self.has_feed_forward = bool(feed_forward)
+        self.roles = ("norm1", "mixer", "norm2", "feed_forward") if self.has_feed_forward else ("norm1", "mixer")
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        s, req = self.streams, {}
+        for q in ("1", "2") if self.has_feed_forward else ("1",):
+            req["in" + q] = WeightRequest((s,), VECTOR)
+            req["out" + q] = WeightRequest((s,), VECTOR)
+            req["mix" + q] = WeightRequest((s, s), VECTOR)
+        return req
+
+    def _sublayer(self, ctx: StepContext, x: torch.Tensor, q: str, norm: Part, call) -> None:
+        n, ws = ctx.n_rows, ctx.workspace
+        u = ws.get("streams_read", n, self.width, torch.float32)
+        y = ws.get("streams_update", n, self.width, torch.float32)
+        kernels.streams_read(x, getattr(self, "in" + q), u, n, self.streams, zero=y)
+        call(LazyNorm(norm, u, n), y)
+        kernels.streams_write(x, getattr(self, "mix" + q), getattr(self, "out" + q), y, n, self.streams)
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        mixer = parts["mixer"]
+        self._sublayer(ctx, x, "1", parts["norm1"],
+                       lambda h, y: mixer.forward_add(ctx, h, y, bindings["mixer"], position))
+        if self.has_feed_forward:
+            feed_forward = parts["feed_forward"]
+            self._sublayer(ctx, x, "2", parts["norm2"], lambda h, y: feed_forward.forward_add(ctx, h, y))

@@ -23,8 +23,10 @@ class TokenEmbedding(Part):
 
     category = "embedding"
 
-    def __init__(self, vocab_size: int, width: int) -> None:
+    def __init__(self, vocab_size: int, width: int, scale: float = 1.0, copies: int = 1) -> None:
         self.vocab_size, self.width = int(vocab_size), int(width)
+        # x0 = table row * scale, written `copies` times side by side (one per residual stream)
+        self.scale, self.copies = float(scale), int(copies)
         self.weight: Optional[torch.Tensor] = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
@@ -32,6 +34,11 @@ class TokenEmbedding(Part):
 
     def forward(self, ctx: StepContext, position: PositionEncoding, x: torch.Tensor) -> None:
         table = position.embedding_table()
+        if self.scale != 1.0 or self.copies != 1:
+            if table is not None:
+                raise ValueError("a scaled or copied embedding takes no position table")
+            kernels.embed_scaled(ctx.token_ids, self.weight, x, ctx.n_rows, self.scale, self.copies)
+            return
         if (residual.usable(ctx, self.width, 1) and self.weight.dtype == torch.bfloat16
                 and (table is None or table.dtype == torch.bfloat16)):
             # a decode-only step of few rows: the rows are looked up by the kernel that reads the
@@ -53,12 +60,19 @@ class LinearHead(Part):
 
     category = "head"
 
-    def __init__(self, vocab_size: int, width: int, tied: bool) -> None:
+    def __init__(self, vocab_size: int, width: int, tied: bool, logit_scale: float = 1.0,
+                 softcap: float = 0.0) -> None:
         self.vocab_size, self.width, self.tied = int(vocab_size), int(width), bool(tied)
+        # logits = softcap * tanh(h W^T * logit_scale / softcap); softcap 0: no cap
+        self.logit_scale, self.softcap = float(logit_scale), float(softcap)
         self.weight: Optional[torch.Tensor] = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
         return {"weight": WeightRequest((self.vocab_size, self.width), MATRIX)}
 
     def forward(self, ctx: StepContext, h: torch.Tensor, logits: torch.Tensor, n_rows: int) -> None:
-        linear(ctx, h, self.weight, None, logits, n_rows, tile_best=ctx.tile_best)
+        if self.logit_scale == 1.0 and self.softcap <= 0.0:
+            linear(ctx, h, self.weight, None, logits, n_rows, tile_best=ctx.tile_best)
+            return
+        linear(ctx, h, self.weight, None, logits, n_rows)
+        kernels.scale_softcap(logits, n_rows, self.logit_scale, self.softcap, fast=not ctx.exact)

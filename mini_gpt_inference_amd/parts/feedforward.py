@@ -7,8 +7,8 @@ from typing import Dict
 import torch
 
 from ..ops import kernels, residual
-from ..ops.linear import LazyNorm, linear, linear_add, packed_weight, plain_residual
-from .base import MATRIX, Part, StepContext, VECTOR, WeightRequest, register_feed_forward
+from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, packed_weight, plain_residual
+from .base import MATRIX, Part, StepContext, TABLE, VECTOR, WeightRequest, register_feed_forward
 
 _ACTIVATIONS = {"gelu_tanh": kernels.EPI_GELU}
 
@@ -82,3 +82,125 @@ class DenseMLP(FeedForward):
         # (a caller that hands over a LazyNorm of x itself knows that x may be left as a sum)
         linear_add(ctx, u, self.proj_weight, self.proj_bias, x, n,
                    may_leave_parts=isinstance(h, LazyNorm) and h.x is x)
+
+
+def _gated(ctx: StepContext, h, in_weight: torch.Tensor, down_weight: torch.Tensor, x: torch.Tensor, n: int,
+           hidden: int) -> None:
+    """x += (silu(h Wgate^T) * (h Wup^T)) Wdown^T with the gate and up matrices stacked in in_weight."""
+    z = ctx.workspace.get("gated_z", n, 2 * hidden, ctx.dtype)
+    linear(ctx, h, in_weight, None, z, n)
+    act = ctx.workspace.get("gated_act", n, hidden, ctx.dtype)
+    kernels.gated_unit(z, act, n, hidden, fast=not ctx.exact)
+    linear_add(ctx, act, down_weight, None, x, n)
+
+
+def _stack_gate_up(part: Part, tensors, gate: str, up: str):
+    """One matrix [2 * hidden, width] from a gate and an up matrix; the two names become views of it."""
+    joint = torch.cat([tensors[gate], tensors[up]], dim=0).contiguous()
+    hidden = tensors[gate].shape[0]
+    views = {gate: joint[:hidden], up: joint[hidden:]}
+    for name, view in views.items():
+        setattr(part, name, view)
+    return joint, views
+
+
+@register_feed_forward("gated_mlp")
+class GatedMLP(FeedForward):
+    """m = (silu(h Wgate^T) * (h Wup^T)) Wdown^T, silu(v) = v sigmoid(v), no biases; the unit's
+    nonlinearity and product in float32."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, hidden: int) -> None:
+        self.width, self.hidden = int(width), int(hidden)
+        self.in_weight = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        return {"gate_weight": WeightRequest((self.hidden, self.width), MATRIX),
+                "up_weight": WeightRequest((self.hidden, self.width), MATRIX),
+                "down_weight": WeightRequest((self.width, self.hidden), MATRIX)}
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        self.in_weight, views = _stack_gate_up(self, tensors, "gate_weight", "up_weight")
+        return views
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor) -> None:
+        plain_residual(ctx, h, x)
+        _gated(ctx, h, self.in_weight, self.down_weight, x, ctx.n_rows, self.hidden)
+
+
+@register_feed_forward("table_experts")
+class TableExperts(FeedForward):
+    """A mixture of gated feed-forwards without a router: row id_t of an integer table [vocab, top]
+    names the experts of token t, each weighted 1 / top; a shared expert (shared_hidden > 0) takes
+    every token and is added.
+
+    The (token, choice) pairs are sorted by expert on the device, every expert multiplies its run
+    of pairs by its own matrices (csrc/hip/experts.hip), and the pairs' outputs are added up per
+    token in the order of the table's columns."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, hidden: int, n_experts: int, top: int, vocab_size: int,
+                 shared_hidden: int = 0) -> None:
+        self.width, self.hidden, self.n_experts, self.top = int(width), int(hidden), int(n_experts), int(top)
+        self.vocab_size, self.shared_hidden = int(vocab_size), int(shared_hidden)
+        if not 0 < self.top <= self.n_experts <= kernels.MAX_EXPERTS:
+            raise ValueError(f"top {self.top} of {self.n_experts} experts: need 0 < top <= experts <= {kernels.MAX_EXPERTS}")
+        self.in_weights = self.down_weights = self.shared_in_weight = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        req = {"table": WeightRequest((self.vocab_size, self.top), TABLE)}
+        for e in range(self.n_experts):
+            req[f"e{e}_gate"] = WeightRequest((self.hidden, self.width), MATRIX)
+            req[f"e{e}_up"] = WeightRequest((self.hidden, self.width), MATRIX)
+            req[f"e{e}_down"] = WeightRequest((self.width, self.hidden), MATRIX)
+        if self.shared_hidden:
+            req["shared_gate"] = WeightRequest((self.shared_hidden, self.width), MATRIX)
+            req["shared_up"] = WeightRequest((self.shared_hidden, self.width), MATRIX)
+            req["shared_down"] = WeightRequest((self.width, self.shared_hidden), MATRIX)
+        return req
+
+    def bind(self, tensors):
+        self.table = tensors["table"]
+        if self.table.dtype != torch.int32:
+            raise ValueError("the experts' table must hold integers")
+        f, views = self.hidden, {}
+        # [experts, 2 * hidden, width] and [experts, width, hidden]: an expert's matrices lie together
+        self.in_weights = torch.stack([torch.cat([tensors[f"e{e}_gate"], tensors[f"e{e}_up"]], dim=0)
+                                       for e in range(self.n_experts)]).contiguous()
+        self.down_weights = torch.stack([tensors[f"e{e}_down"] for e in range(self.n_experts)]).contiguous()
+        for e in range(self.n_experts):
+            views[f"e{e}_gate"], views[f"e{e}_up"] = self.in_weights[e, :f], self.in_weights[e, f:]
+            views[f"e{e}_down"] = self.down_weights[e]
+        if self.shared_hidden:
+            self.shared_down = tensors["shared_down"]
+            self.shared_in_weight, shared = _stack_gate_up(self, tensors, "shared_gate", "shared_up")
+            views.update(shared)
+        return views
+
+    def token_matrix_elements(self) -> int:
+        """Matrix elements one token goes through: its `top` experts and the shared one."""
+        return 3 * self.width * (self.top * self.hidden + self.shared_hidden)
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor) -> None:
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        hn = as_tensor(ctx, h)
+        slots = kernels.expert_slots(n, self.top, self.n_experts)
+        slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
+        slot_pair = ws.get("expert_slot_pair", slots, 1, torch.int32).view(-1)
+        tile_expert = ws.get("expert_tile", slots // kernels.EXPERT_TILE, 1, torch.int32).view(-1)
+        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair, tile_expert)
+        z = ws.get("expert_z", slots, 2 * self.hidden, ctx.dtype)
+        kernels.grouped_linear(hn, slot_token, self.in_weights, tile_expert, slot_token, z, None, slots)
+        act = ws.get("expert_act", slots, self.hidden, ctx.dtype)
+        kernels.gated_unit(z, act, slots, self.hidden, fast=not ctx.exact)
+        pair_out = ws.get("expert_pair_out", n * self.top, self.width, torch.float32)
+        kernels.grouped_linear(act, None, self.down_weights, tile_expert, slot_token, pair_out, slot_pair, slots)
+        if self.shared_hidden:
+            _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
+        kernels.expert_combine(pair_out, x, n, self.top, 1.0 / self.top)

@@ -136,3 +136,92 @@ class PagedCausalAttention(Mixer):
         attention_ops.paged_attention(ctx, qkv, y, k_pool, v_pool, group, self.n_head, self.scale, self.window)
         linear_add(ctx, y, self.proj_weight, self.proj_bias, x, n,
                    may_leave_parts=isinstance(h, LazyNorm) and h.x is x)
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    """Attention whose keys and values are made from one small latent per token, which is all the
+    cache keeps (one joint tensor per page), without a position signal.
+
+    c = rms_norm(h Wdkv^T) * gain, [rank], stored into the pages.  Per head a: q_a = h Wq_a^T [D],
+    k_a = Wuk_a c [D], v_a = Wuv_a c [E]; S = (q_a . k_a) * scale over the keys at positions
+    p - window < j <= p (window 0: all j <= p); softmax in float32 with one more term exp(sink_a) in
+    the denominator that has no value; y = concat_a(P v_a) * sigmoid(h Wg^T); out = y Wo^T, added
+    into the residual.
+
+    The kernels never make k_a and v_a: (q_a . Wuk_a c) = (Wuk_a^T q_a) . c, so the queries are
+    folded onto the latent basis (one product per head), attention runs with one key/value head of
+    size `rank` that every query head shares, and its output sum_j P_j c_j is unfolded by Wuv_a
+    afterwards.  A layer with makes_latent=False has no Wdkv: it reads the pages that another run
+    of the same step wrote (LayerRun.reads_cache_of), with its own Wuk, Wuv, window and the rest."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, n_head: int, head_dim: int, value_dim: int, rank: int, scale: float,
+                 window: int = 0, eps: float = 1e-6, makes_latent: bool = True) -> None:
+        self.width, self.n_head, self.head_dim = int(width), int(n_head), int(head_dim)
+        self.value_dim, self.rank = int(value_dim), int(rank)
+        self.scale, self.window, self.eps = float(scale), int(window), float(eps)
+        self.makes_latent = bool(makes_latent)
+        if not 0 < self.rank <= 256:
+            raise ValueError(f"latent size {self.rank}: the attention kernels take up to 256")
+        self.q_width, self.g_width = self.n_head * self.head_dim, self.n_head * self.value_dim
+        self.in_weight = self.uk_folded = self.uv_heads = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        req = {"q_weight": WeightRequest((self.q_width, self.width), MATRIX),
+               "gate_weight": WeightRequest((self.g_width, self.width), MATRIX),
+               "uk_weight": WeightRequest((self.q_width, self.rank), MATRIX),
+               "uv_weight": WeightRequest((self.g_width, self.rank), MATRIX),
+               "sink": WeightRequest((self.n_head,), VECTOR),
+               "out_weight": WeightRequest((self.width, self.g_width), MATRIX)}
+        if self.makes_latent:
+            req["dkv_weight"] = WeightRequest((self.rank, self.width), MATRIX)
+            req["dkv_norm"] = WeightRequest((self.rank,), VECTOR)
+        return req
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        # the products that read h as one: queries, gate and (where this layer makes it) the latent
+        names = ["q_weight", "gate_weight"] + (["dkv_weight"] if self.makes_latent else [])
+        self.in_weight = torch.cat([tensors[n] for n in names], dim=0).contiguous()
+        views, at = {}, 0
+        for n in names:
+            rows = tensors[n].shape[0]
+            views[n] = self.in_weight[at:at + rows]
+            setattr(self, n, views[n])
+            at += rows
+        # per head: Wuk_a^T as [rank, D] (so that folding a query is a product with a matrix stored
+        # [out, in]) and Wuv_a as [E, rank]
+        self.uk_folded = self.uk_weight.view(self.n_head, self.head_dim, self.rank).transpose(1, 2).contiguous()
+        self.uv_heads = self.uv_weight.view(self.n_head, self.value_dim, self.rank)
+        self.uk_weight = self.uk_folded.transpose(1, 2)
+        views["uk_weight"] = self.uk_weight
+        return views
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(1, self.rank, self.window, joint=True)
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        if binding.writes != self.makes_latent:
+            raise ValueError("a latent-attention layer writes the latent cache exactly when it has the matrix that makes it")
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        fast = not ctx.exact
+        z = ws.get("latent_in", n, self.in_weight.shape[0], ctx.dtype)
+        linear(ctx, h, self.in_weight, None, z, n)
+        group = ctx.groups[binding.group]
+        pool = group.k_pools[binding.index]
+        if self.makes_latent:
+            kernels.rms_norm_store(z[:, self.q_width + self.g_width:], self.dkv_norm, self.eps, pool,
+                                   group.slot_mapping, n)
+        q_lat = ws.get("latent_q", n, self.n_head * self.rank, ctx.dtype)
+        kernels.heads_linear(z, self.uk_folded, q_lat, n, fast=fast)
+        o_lat = ws.get("latent_o", n, self.n_head * self.rank, ctx.dtype)
+        attention_ops.paged_attention(ctx, q_lat, o_lat, pool, pool, group, self.n_head, self.scale, self.window,
+                                      sinks=self.sink)
+        y = ws.get("attn_out", n, self.g_width, ctx.dtype)
+        kernels.heads_linear(o_lat, self.uv_heads, y, n, gate=z[:, self.q_width:self.q_width + self.g_width], fast=fast)
+        linear_add(ctx, y, self.out_weight, None, x, n)

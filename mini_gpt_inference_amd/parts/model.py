@@ -13,7 +13,7 @@ from typing import Dict, List, Mapping, Optional, Tuple
 
 import torch
 
-from ..ops import residual
+from ..ops import kernels, residual
 from ..ops.linear import LazyNorm
 from . import block as _block  # noqa: F401  (registers the parts)
 from . import embedding as _embedding  # noqa: F401
@@ -79,6 +79,9 @@ class ModelSpec:
     final_norm: PartSpec
     head: PartSpec
     max_positions: Optional[int] = None
+    # residual streams a token has between the layers (hyper-connections); the residual buffer is
+    # [rows, streams * width], the embedding fills every stream and their sum goes to the final norm
+    streams: int = 1
     # (duplicate name, tensor it must equal): names a checkpoint may carry beside the tensor they alias
     tied_aliases: Tuple[Tuple[str, str], ...] = ()
 
@@ -88,8 +91,9 @@ class CacheGroupSpec:
     """Runs whose mixers keep the same kind of pages share a page table and a pool geometry."""
     n_kv_head: int
     head_dim: int
-    window: int
+    window: int        # what the pages must keep: the widest window among the runs that write or read them
     n_pools: int       # caches (one per writing run) in the group
+    joint: bool = False   # keys and values are one tensor
 
 
 @dataclass
@@ -111,6 +115,7 @@ class KVRun:
     n_kv_head: int
     head_dim: int
     window: int
+    tensors: int = 2      # cached tensors a key position costs: keys and values, or one joint latent
 
 
 @dataclass(frozen=True)
@@ -132,7 +137,7 @@ class ModelCost:
         for run in self.kv_runs:
             for c in context_lens:
                 reach = min(c, run.window) if run.window else c
-                kv += reach * 2 * run.n_kv_head * run.head_dim * cache_itemsize
+                kv += reach * run.tensors * run.n_kv_head * run.head_dim * cache_itemsize
         return self.whole_tensor_bytes + n_tokens * self.table_row_bytes + kv
 
     def prompt_flops(self, prompt_lens, n_logit_rows: int) -> float:
@@ -189,6 +194,7 @@ class DecoderModel:
         pairs = [(self.embedding, self.spec.embedding), (self.position, self.spec.position)]
         for layer, ls in zip(self.layers, self.spec.layers):
             pairs += [(layer.parts[role], part_spec) for role, (_, part_spec) in ls.parts.items()]
+            pairs.append((layer.arrangement, ls.arrangement))      # an arrangement may have tensors of its own
         pairs += [(self.final_norm, self.spec.final_norm), (self.head, self.spec.head)]
         return pairs
 
@@ -210,7 +216,9 @@ class DecoderModel:
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self._bound = {name: tensors[name] for name in self.weight_requests()}
         for part, spec in self._named_parts():
-            part.bind({local: tensors[spec.weights[local]] for local in part.weight_requests()})
+            replaced = part.bind({local: tensors[spec.weights[local]] for local in part.weight_requests()})
+            for local, view in (replaced or {}).items():
+                self._bound[spec.weights[local]] = view
 
     def weight_bytes(self) -> Tuple[int, int]:
         """(bytes of the tensors as loaded, bytes of the copies derived from them since: matrices
@@ -242,6 +250,8 @@ class DecoderModel:
         row_bytes = sum(size(name) // bound[name].shape[0] for name in by_row)
 
         def matrices(part: Part) -> int:
+            if hasattr(part, "token_matrix_elements"):      # a part whose tokens go through some of its matrices only
+                return int(part.token_matrix_elements())
             total = 0
             for req in part.weight_requests().values():
                 if req.role == "matrix":
@@ -259,37 +269,56 @@ class DecoderModel:
                 need = part.cache_need() if hasattr(part, "cache_need") else None
                 if isinstance(need, KVNeed):
                     kv_runs.append(KVRun(int(getattr(part, "n_head", need.n_kv_head)), need.n_kv_head,
-                                         need.head_dim, need.window))
+                                         need.head_dim, need.window, 1 if need.joint else 2))
         return ModelCost(sum(size(name) for name in whole), row_bytes, run_elements, matrices(self.head),
                          tuple(kv_runs))
 
     # ------------------------------------------------------------------ cache
     def _plan_cache(self) -> CacheLayout:
         groups: List[CacheGroupSpec] = []
-        keys: List[Tuple[int, int, int]] = []
+        keys: List[Tuple[int, int, int, bool]] = []
         state_numels: List[int] = []
         run_bindings: List[Dict[str, CacheBinding]] = []
+
+        def need_of(run_index: int, role: str):
+            parts = self.layers[self.spec.order[run_index].layer].parts
+            return parts[role].cache_need() if role in parts else None
+
+        def same_pages(a, b) -> bool:
+            return (isinstance(a, KVNeed) and isinstance(b, KVNeed)
+                    and (a.n_kv_head, a.head_dim, a.joint) == (b.n_kv_head, b.head_dim, b.joint))
+
+        # What a writing run's pages must keep: the widest window among itself and the runs that read
+        # its cache (each masks with its own window; 0, all keys, is the widest).
+        reach: Dict[Tuple[int, str], int] = {}
         for i, run in enumerate(self.spec.order):
-            layer, layer_spec = self.layers[run.layer], self.spec.layers[run.layer]
+            for role in self.spec.layers[run.layer].roles("mixer"):
+                need = need_of(i, role)
+                if not isinstance(need, KVNeed):
+                    continue
+                key = (i if run.reads_cache_of is None else run.reads_cache_of, role)
+                seen = reach.get(key)
+                reach[key] = need.window if seen is None else (0 if 0 in (seen, need.window) else max(seen, need.window))
+
+        for i, run in enumerate(self.spec.order):
+            layer_spec = self.spec.layers[run.layer]
             bindings: Dict[str, CacheBinding] = {}
             for role in layer_spec.roles("mixer"):
-                need = layer.parts[role].cache_need()
+                need = need_of(i, role)
                 if run.reads_cache_of is not None:
-                    src_run = self.spec.order[run.reads_cache_of]
                     src = run_bindings[run.reads_cache_of].get(role)
-                    src_need = (self.layers[src_run.layer].parts[role].cache_need()
-                                if role in self.layers[src_run.layer].parts else None)
-                    if src is None or need != src_need or src.kind != "kv":
+                    if src is None or src.kind != "kv" or not src.writes \
+                            or not same_pages(need, need_of(run.reads_cache_of, role)):
                         raise ValueError(f"run {i} cannot read the cache of run {run.reads_cache_of}: different needs")
                     bindings[role] = CacheBinding("kv", src.group, src.index, writes=False)
                 elif isinstance(need, KVNeed):
-                    key = (need.n_kv_head, need.head_dim, need.window)
+                    key = (need.n_kv_head, need.head_dim, reach[(i, role)], need.joint)
                     if key not in keys:
                         keys.append(key)
-                        groups.append(CacheGroupSpec(need.n_kv_head, need.head_dim, need.window, 0))
+                        groups.append(CacheGroupSpec(key[0], key[1], key[2], 0, key[3]))
                     g = keys.index(key)
                     bindings[role] = CacheBinding("kv", g, groups[g].n_pools, writes=True)
-                    groups[g] = CacheGroupSpec(*key, groups[g].n_pools + 1)
+                    groups[g] = CacheGroupSpec(key[0], key[1], key[2], groups[g].n_pools + 1, key[3])
                 elif isinstance(need, StateNeed):
                     bindings[role] = CacheBinding("state", -1, len(state_numels), writes=True)
                     state_numels.append(int(need.numel))
@@ -321,7 +350,8 @@ class DecoderModel:
         the last position only)."""
         n = ctx.n_rows
         ws = ctx.workspace
-        x = ws.get("residual", n, self.spec.width, torch.float32)
+        streams = self.spec.streams
+        x = ws.get("residual", n, streams * self.spec.width, torch.float32)
         ctx.pending = None
         self.embedding.forward(ctx, self.position, x)
         for run, bindings in zip(self.spec.order, self.cache_layout.run_bindings):
@@ -329,6 +359,11 @@ class DecoderModel:
             if not layer.arrangement.takes_pending_residual:
                 residual.settle(ctx, x, n)
             layer.arrangement.run(ctx, x, layer.parts, bindings, self.position)
+        if streams > 1:
+            # the streams' sum is what the final norm reads
+            total = ws.get("residual_sum", n, self.spec.width, torch.float32)
+            kernels.streams_read(x, None, total, n, streams)
+            x = total
         m = ctx.m_rows
         # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
         # whatever the vocabulary's size (50257 is odd)

@@ -28,9 +28,18 @@ def random_tensors(config, seed: int, dtype: torch.dtype = torch.bfloat16, std_s
     gen.manual_seed(int(seed))
     tensors: Dict[str, torch.Tensor] = {}
     for name, shape, rule, scale in arch.init_plan(config):
+        if rule == "distinct":
+            # an integer table: every row names shape[1] different values below `scale`
+            order = torch.rand((shape[0], int(scale)), generator=gen).argsort(dim=1)
+            tensors[name] = order[:, :shape[1]].to(torch.int32).contiguous()
+            continue
         t = torch.empty(shape, dtype=torch.float32).normal_(0.0, scale * std_scale, generator=gen)
         if rule == "gain":
             t += 1.0
+        elif rule == "around":          # values near `scale`
+            t = t * 0.25 + scale
+        elif rule == "identity":        # a square matrix near the identity
+            t += torch.eye(shape[0])
         elif rule != "normal":
             raise ValueError(f"unknown init rule {rule!r} for {name}")
         tensors[name] = t.to(dtype).contiguous()
