@@ -24,7 +24,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
-    int n_kv_head, int head_dim, int page_size, float scale, int window) {
+    int n_kv_head, int head_dim, int page_size, float scale, int window, const float* __restrict__ sinks) {
   __shared__ float q_s[AD_MAX_DPL * 64];
   __shared__ float p_s[AD_WAVES][64];
   __shared__ int page_s[AD_WAVES][64];
@@ -116,7 +116,11 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
   if (wave == 0) {
     float mx = m_s[0];
     for (int w = 1; w < AD_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
-    float lt = 0.f;
+    // a sink is one more term of the denominator, with no value
+    const bool sunk = sinks != nullptr;
+    const float sink = sunk ? sinks[h] : 0.f;
+    if (sunk) mx = fmaxf(mx, sink);
+    float lt = sunk ? __expf(sink - mx) : 0.f;
     float f[AD_WAVES];
     for (int w = 0; w < AD_WAVES; ++w) {
       f[w] = (m_s[w] == -INFINITY) ? 0.f : __expf(m_s[w] - mx);
@@ -139,7 +143,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    hipStream_t stream) {
+    const float* sinks, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
@@ -149,7 +153,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
   hipLaunchKernelGGL(paged_attention_split_kernel, dim3(n_tokens, n_head), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,
                      block_tables, max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim,
-                     page_size, scale, window);
+                     page_size, scale, window, sinks);
   return mgpt_last_error();
 }
 
@@ -165,7 +169,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
-    int n_kv_head, int page_size, float scale, int window) {
+    int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   __shared__ float m_s[AD_WAVES], l_s[AD_WAVES];
@@ -275,7 +279,10 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
   if (tid < D) {
     float mx = m_s[0];
     for (int w = 1; w < AD_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
-    float lt = 0.f, a = 0.f;
+    const bool sunk = sinks != nullptr;
+    const float sink = sunk ? sinks[h] : 0.f;
+    if (sunk) mx = fmaxf(mx, sink);
+    float lt = sunk ? __expf(sink - mx) : 0.f, a = 0.f;
     for (int w = 0; w < AD_WAVES; ++w) {
       const float f = (m_s[w] == -INFINITY) ? 0.f : __expf(m_s[w] - mx);
       lt += l_s[w] * f;
@@ -289,7 +296,7 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    hipStream_t stream) {
+    const float* sinks, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
@@ -300,7 +307,7 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
 #define AD_LAUNCH(DD)                                                                                   \
   hipLaunchKernelGGL(paged_attention_split_fast_kernel<DD>, grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,       \
-                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window)
+                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks)
   switch (head_dim) {
     case 16: AD_LAUNCH(16); break;
     case 32: AD_LAUNCH(32); break;

@@ -10,17 +10,17 @@ extern "C" {
 int mgpt_paged_attention_split_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int*
     q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    hipStream_t stream);
+    const float* sinks, hipStream_t stream);
 // attention_decode.hip
 int mgpt_paged_attention_split_fast_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool,
     const void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const
     int* q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    hipStream_t stream);
+    const float* sinks, hipStream_t stream);
 // attention_decode_wide.hip
 int mgpt_paged_attention_decode_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int*
     cu_q, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale,
-    int window, int identity, hipStream_t stream);
+    int window, int identity, const float* sinks, hipStream_t stream);
 // attention_generic.hip
 int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, void* kpool, void* vpool, const
     int* slot_mapping, int n_tokens, int n_kv_head, int head_dim, int page_size, hipStream_t stream);
@@ -33,7 +33,7 @@ int mgpt_paged_attention_generic(const void* q, long ldq, void* out, long ldo, c
 int mgpt_prefill_attention_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req, int
     max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int
-    single_below, hipStream_t stream);
+    single_below, const float* sinks, hipStream_t stream);
 // embed_norm.hip
 int mgpt_embed(const int* ids, const int* pos, const void* tok, const void* postab, float* x, int n_tokens,
     int width, int table_dtype, hipStream_t stream);

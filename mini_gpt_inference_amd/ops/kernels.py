@@ -484,7 +484,7 @@ def linear_skinny_partials(n_rows: int, n_out: int, k_dim: int, has_ln: bool, ep
 def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                                block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                                q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
-                               window: int = 0, fast: bool = True) -> bool:
+                               window: int = 0, fast: bool = True, sinks: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused.
     fast=False keeps to the variant that takes every head size."""
     if q.dtype != torch.bfloat16:
@@ -493,13 +493,14 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
     if head_dim % 8 != 0 or head_dim > 256 or k_pool.data_ptr() % 16 != 0:
         return False
+    _need_sinks(sinks, n_head)
     fn = library.kernels().mgpt_paged_attention_split_bf16
     if fast and head_dim in (16, 32, 64, 128) and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0:
         fn = library.kernels().mgpt_paged_attention_split_fast_bf16   # all loads 16 bytes wide
     rc = fn(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _stream())
+        page_size, float(scale), int(window), _ptr(sinks), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_split_bf16")
@@ -509,7 +510,8 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
 def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                                 block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor,
                                 n_tokens: int, n_head: int, scale: float, window: int = 0,
-                                identity: bool = False, cu_q: Optional[torch.Tensor] = None) -> bool:
+                                identity: bool = False, cu_q: Optional[torch.Tensor] = None,
+                                sinks: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention for single tokens (one query per request and step), keys split over eight
     waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
     padded token; identity=True promises q_req[n] in (n, -1).  With cu_q (the requests' token offsets;
@@ -534,6 +536,7 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
           "block_tables must be dense int32 [requests, blocks]")
     _need_i32("positions", positions, n_tokens)
     _need_i32("q_req", q_req, n_tokens)
+    _need_sinks(sinks, n_head)
     if identity:
         _need(block_tables.shape[0] >= n_tokens, "a decode-only step needs a block table row per token")
         _need(cu_q is None, "cu_q is for steps that are not decode-only")
@@ -543,7 +546,7 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     rc = library.kernels().mgpt_paged_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(positions), _ptr(q_req), _ptr(cu_q), n_tokens, n_head, n_kv_head, head_dim, page_size,
-        num_pages, float(scale), int(window), 1 if identity else 0, _stream())
+        num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_decode_bf16")
@@ -653,7 +656,7 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
                            max_q_len: int, n_head: int, scale: float, window: int = 0,
-                           single_below: int = 0) -> bool:
+                           single_below: int = 0, sinks: Optional[torch.Tensor] = None) -> bool:
     """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
     rows of q from cu_q; a request may bring none).  Requests that bring exactly one token, and that
     among the step's first `single_below` tokens, are left to another kernel.  False when it does
@@ -676,10 +679,11 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
           and block_tables.shape[0] >= n_req, "block_tables must be dense int32 [>=requests, max_blocks]")
     _need_i32("cu_q", cu_q, n_req + 1)
     _need_i32("seq_lens", seq_lens, n_req)
+    _need_sinks(sinks, n_head)
     rc = library.kernels().mgpt_prefill_attention_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), int(single_below), _stream())
+        page_size, float(scale), int(window), int(single_below), _ptr(sinks), _stream())
     if rc == -2:
         return False
     _check(rc, "prefill_attention_bf16")
