@@ -119,6 +119,14 @@ def _mlp_from_json(i: int, mlp: Optional[Mapping[str, Any]]) -> Optional[FeedFor
     raise ConfigError(f"layer {i}: unknown feed-forward kind {kind!r}")
 
 
+def _softcap(value: Any) -> float:
+    if value is None:
+        return 0.0          # no cap
+    if not float(value) > 0.0:
+        raise ConfigError(f"logit_softcap must be positive, got {value!r}")
+    return float(value)
+
+
 def config_from_json(raw: Mapping[str, Any]) -> ViperaxConfig:
     layers: List[LayerConfig] = []
     if not isinstance(raw.get("layers"), list) or not raw["layers"]:
@@ -131,7 +139,7 @@ def config_from_json(raw: Mapping[str, Any]) -> ViperaxConfig:
         layers=tuple(layers), norm_eps=float(raw["norm"]["eps"]),
         embedding_scale=float((raw.get("embedding") or {}).get("scale", 1.0)),
         streams=None if streams is None else _positive("streams", streams),
-        logit_scale=float(raw.get("logit_scale", 1.0)), logit_softcap=float(raw.get("logit_softcap", 0.0)))
+        logit_scale=float(raw.get("logit_scale", 1.0)), logit_softcap=_softcap(raw.get("logit_softcap")))
 
 
 def config_to_json(cfg: ViperaxConfig) -> Dict[str, Any]:
@@ -155,7 +163,9 @@ def config_to_json(cfg: ViperaxConfig) -> Dict[str, Any]:
         layers.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
     out: Dict[str, Any] = {"architecture": NAME, "vocab": cfg.vocab, "width": cfg.width, "layers": layers,
                            "norm": {"eps": cfg.norm_eps}, "embedding": {"scale": cfg.embedding_scale},
-                           "logit_scale": cfg.logit_scale, "logit_softcap": cfg.logit_softcap}
+                           "logit_scale": cfg.logit_scale}
+    if cfg.logit_softcap > 0.0:
+        out["logit_softcap"] = cfg.logit_softcap
     if cfg.streams is not None:
         out["streams"] = cfg.streams
     return out

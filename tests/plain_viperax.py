@@ -28,6 +28,22 @@ def read_model_folder(path: str) -> Tuple[dict, Dict[str, torch.Tensor]]:
     return cfg, tensors
 
 
+# With ROUNDING set to torch.bfloat16 every matrix product takes operands rounded to that format and
+# its result is rounded to it too, as a kernel that computes "in bfloat16 with 32-bit accumulation"
+# does.  The difference between the two modes is the size of what rounding alone does to the
+# logits: the tests' bound for the engine's bfloat16 path is a multiple of it.
+ROUNDING = None
+
+
+def _r(x: torch.Tensor) -> torch.Tensor:
+    return x if ROUNDING is None else x.to(ROUNDING).to(torch.float32)
+
+
+def lin(h: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """w h for every row of h, w stored [out, in]."""
+    return _r(_r(h) @ _r(w).T)
+
+
 # ---------------------------------------------------------------- norms
 def layer_norm(x: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
     """(x - mean) / sqrt(var + eps) * gain; var is the mean squared deviation; no bias."""
@@ -49,7 +65,7 @@ def silu(z: torch.Tensor) -> torch.Tensor:
 
 def gated_mlp(h: torch.Tensor, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor) -> torch.Tensor:
     """down (silu(gate h) * (up h)), matrices stored [out, in]."""
-    return (silu(h @ gate.T) * (h @ up.T)) @ down.T
+    return lin(silu(lin(h, gate)) * lin(h, up), down)
 
 
 def table_moe(h: torch.Tensor, token_ids: List[int], table: torch.Tensor, experts: List[Tuple[torch.Tensor, ...]],
@@ -69,31 +85,39 @@ def table_moe(h: torch.Tensor, token_ids: List[int], table: torch.Tensor, expert
 # ---------------------------------------------------------------- latent attention
 def latents(h: torch.Tensor, w_dkv: torch.Tensor, gain: torch.Tensor, eps: float) -> torch.Tensor:
     """What a layer remembers of every token: the RMS-normed down-projection, [T, R]."""
-    return rms_norm(h @ w_dkv.T, gain, eps)
+    return rms_norm(lin(h, w_dkv), gain, eps)
+
+
+def sink_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sink: Optional[torch.Tensor], scale: float,
+                   window: int) -> torch.Tensor:
+    """q [T, H, D], k [T, H, D], v [T, H, E] of one sequence -> [T, H, E].  Query i sees key j when
+    0 <= i - j < window (window 0: every j <= i).  The softmax's denominator has one more term per
+    head, exp(sink), with no value (sink None: the ordinary softmax)."""
+    T, heads = q.shape[0], q.shape[1]
+    out = torch.zeros(T, heads, v.shape[-1], dtype=q.dtype)
+    for i in range(T):
+        lo = 0 if window <= 0 else max(0, i - window + 1)
+        for a in range(heads):
+            s = (k[lo:i + 1, a] @ q[i, a]) * scale                 # [keys]
+            top = float(s.max()) if sink is None else max(float(s.max()), float(sink[a]))
+            e = torch.exp(s - top)
+            denom = e.sum() + (0.0 if sink is None else math.exp(float(sink[a]) - top))
+            out[i, a] = (e / denom) @ v[lo:i + 1, a]
+    return out
 
 
 def latent_attention(h: torch.Tensor, c: torch.Tensor, w_q: torch.Tensor, w_uk: torch.Tensor, w_uv: torch.Tensor,
                      sink: torch.Tensor, w_g: torch.Tensor, w_o: torch.Tensor, heads: int, scale: float,
                      window: int) -> torch.Tensor:
     """Queries from h, keys and values from the latents c (this layer's or another's), no position
-    signal.  Query i sees key j when 0 <= i - j < window (window 0: every j <= i).  The softmax's
-    denominator has one more term per head, exp(sink), with no value.  The heads' outputs are
-    gated by sigmoid(w_g h) before w_o."""
+    signal; sink_attention; the heads' outputs are gated by sigmoid(w_g h) before w_o."""
     T = h.shape[0]
-    q = (h @ w_q.T).view(T, heads, -1)
-    k = (c @ w_uk.T).view(T, heads, -1)
-    v = (c @ w_uv.T).view(T, heads, -1)
-    out = torch.zeros(T, heads, v.shape[-1])
-    for i in range(T):
-        lo = 0 if window <= 0 else max(0, i - window + 1)
-        for a in range(heads):
-            s = (k[lo:i + 1, a] @ q[i, a]) * scale                 # [keys]
-            top = max(float(s.max()), float(sink[a]))
-            e = torch.exp(s - top)
-            denom = e.sum() + math.exp(float(sink[a]) - top)
-            out[i, a] = (e / denom) @ v[lo:i + 1, a]
-    gate = 1.0 / (1.0 + torch.exp(-(h @ w_g.T)))
-    return (out.reshape(T, -1) * gate) @ w_o.T
+    q = lin(h, w_q).view(T, heads, -1)
+    k = lin(c, w_uk).view(T, heads, -1)
+    v = lin(c, w_uv).view(T, heads, -1)
+    out = _r(sink_attention(q, k, v, sink, scale, window))
+    gate = 1.0 / (1.0 + torch.exp(-lin(h, w_g)))
+    return lin(out.reshape(T, -1) * gate, w_o)
 
 
 # ---------------------------------------------------------------- hyper-connections
@@ -142,7 +166,7 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int]) -> Tuple[t
     """Logits [T, vocab] of one sequence, and the residual stream (the streams' sum) after every
     layer, [layers, T, W]."""
     eps = float(cfg["norm"]["eps"])
-    x0 = w["embed"][torch.tensor(tokens)] * float(cfg["embedding"]["scale"])
+    x0 = w["embed"][torch.tensor(tokens)] * float(cfg.get("embedding", {}).get("scale", 1.0))
     hyper = "streams" in cfg
     streams = x0[None].repeat(int(cfg["streams"]), 1, 1) if hyper else x0[None].clone()
     kept: Dict[int, torch.Tensor] = {}
@@ -160,9 +184,11 @@ def forward(cfg: dict, w: Dict[str, torch.Tensor], tokens: List[int]) -> Tuple[t
                 streams = streams + fn(layer_norm(streams[0], w[f"l{i}.norm{q}"], eps))[None]
         after.append(streams.sum(dim=0))
     x = streams.sum(dim=0)
-    logits = layer_norm(x, w["final.norm"], eps) @ w["head"].T * float(cfg["logit_scale"])
-    cap = float(cfg["logit_softcap"])
-    logits = cap * torch.tanh(logits / cap)
+    logits = _r(_r(layer_norm(x, w["final.norm"], eps)) @ _r(w["head"]).T).to(torch.float32) \
+        * float(cfg.get("logit_scale", 1.0))
+    if "logit_softcap" in cfg:
+        cap = float(cfg["logit_softcap"])
+        logits = cap * torch.tanh(logits / cap)
     return logits, torch.stack(after)
 
 

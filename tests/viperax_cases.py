@@ -1,0 +1,91 @@
+"""Small Viperax configurations and model folders with random weights for the tests.
+
+The configurations differ from each other in every size and option: streams (several, one, none),
+heads (also one), query/key size against value size, latent sizes that the bfloat16 tile kernel
+takes (32, 64) and that it does not (40, 24), windows (none, 1, a few tokens, longer than the
+prompts), layers that read another layer's latents through a longer or a shorter window than the
+layer that writes them, feed-forwards (none, dense, experts with top 1 and 2, with and without a
+shared expert), logit scale and cap."""
+
+from __future__ import annotations
+
+import os
+from typing import Callable, Dict, Optional
+
+import torch
+from safetensors.torch import save_file
+
+from mini_gpt_inference_amd.config.model_config import write_config_json
+from mini_gpt_inference_amd.models import viperax
+from mini_gpt_inference_amd.weights.random_init import random_tensors
+
+
+def _mixer(heads, dim, vdim, rank, scale, window=None, kv_from=None):
+    m = {"heads": heads, "dim": dim, "vdim": vdim, "kv_rank": rank, "scale": scale}
+    if window is not None:
+        m["mask"] = {"size": window}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return m
+
+
+def _layer(mixer, mlp):
+    return {"type": "latent_attention", "mixer": mixer, "mlp": mlp}
+
+
+def _moe(ff, experts, top, shared=None):
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "top": top}}
+    if shared:
+        mlp["shared"] = {"ff": shared}
+    return mlp
+
+
+RAW: Dict[str, dict] = {
+    # several streams; a layer that reads layer 1's latents through a longer window than layer 1's own,
+    # one without a feed-forward, one that reads layer 0's without any mask
+    "P": {"architecture": "Viperax", "vocab": 131, "width": 64, "streams": 2, "norm": {"eps": 1e-5},
+          "embedding": {"scale": 8.0}, "logit_scale": 0.5, "logit_softcap": 10.0,
+          "layers": [_layer(_mixer(2, 16, 32, 32, 0.3, window=9), {"kind": "dense", "ff": 48}),
+                     _layer(_mixer(2, 16, 32, 32, 0.3, window=20), _moe(24, 5, 2, shared=40)),
+                     _layer(_mixer(4, 8, 16, 32, 0.4, window=33, kv_from=1), None),
+                     _layer(_mixer(2, 16, 32, 32, 0.3, kv_from=0), _moe(16, 3, 1))]},
+    # one stream with hyper-connection tensors, one head, top 1 of 2, a window of one token, a latent
+    # size (40) that only the split and the general kernels take, no cap on the logits
+    "Q": {"architecture": "Viperax", "vocab": 77, "width": 48, "streams": 1, "norm": {"eps": 1e-6},
+          "embedding": {"scale": 1.0}, "logit_scale": 2.0,
+          "layers": [_layer(_mixer(1, 24, 8, 40, 0.2, window=1), _moe(32, 2, 1)),
+                     _layer(_mixer(3, 8, 24, 40, 0.35, window=5), {"kind": "dense", "ff": 20}),
+                     _layer(_mixer(1, 24, 8, 40, 0.2, window=3, kv_from=1), {"kind": "dense", "ff": 36})]},
+    # no hyper-connections at all (no `streams` key), no masks, a latent of 64, three streams' worth of
+    # nothing: the plain pre-norm residual; top 3 of 4 with a shared expert
+    "R": {"architecture": "Viperax", "vocab": 203, "width": 96, "norm": {"eps": 1e-4},
+          "embedding": {"scale": 3.0}, "logit_scale": 1.0, "logit_softcap": 30.0,
+          "layers": [_layer(_mixer(3, 32, 16, 64, 0.18), _moe(40, 4, 3, shared=24)),
+                     _layer(_mixer(2, 16, 48, 64, 0.25, kv_from=0), {"kind": "dense", "ff": 112})]},
+    # three streams, a latent of 24 (the general kernel only), windows longer than most prompts
+    "S": {"architecture": "Viperax", "vocab": 59, "width": 40, "streams": 3, "norm": {"eps": 1e-5},
+          "embedding": {"scale": 6.0}, "logit_scale": 0.25, "logit_softcap": 5.0,
+          "layers": [_layer(_mixer(2, 12, 20, 24, 0.3, window=70), {"kind": "dense", "ff": 56}),
+                     _layer(_mixer(2, 12, 20, 24, 0.3, window=4, kv_from=0), _moe(8, 6, 2))]},
+}
+SEEDS = {"P": 3, "Q": 4, "R": 5, "S": 6}
+STD_SCALE = {"P": 1.5, "Q": 1.5, "R": 1.5, "S": 1.5}
+
+
+def config(name: str):
+    return viperax.config_from_json(RAW[name])
+
+
+def write_model(path: str, name: str, edit: Optional[Callable[[Dict[str, torch.Tensor]], None]] = None) -> str:
+    cfg = config(name)
+    tensors = random_tensors(cfg, SEEDS[name], torch.bfloat16, STD_SCALE[name])
+    # sinks large enough to matter: a kernel that leaves one out, or counts it twice, shows
+    for key in tensors:
+        if key.endswith(".sink"):
+            tensors[key] = (tensors[key].float() * 2.0 + 1.0).to(torch.bfloat16)
+    if edit is not None:
+        edit(tensors)
+    os.makedirs(path, exist_ok=True)
+    write_config_json(path, cfg)
+    save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(path, "model.safetensors"))
+    return path
