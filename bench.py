@@ -35,7 +35,9 @@ REFERENCE_DECODE_B8 = 1671.8               # tok/s, the reference's own figure (
 def raw_model_config(args, **override):
     """The config.json dict of the model to measure: the file --model-config names (any registered
     architecture), or the reference's 50.9M model with the sizes of the command line."""
-    if args.model_config:
+    if getattr(args, "raw_config", None):
+        raw = json.loads(json.dumps(args.raw_config))
+    elif args.model_config:
         with open(args.model_config, encoding="utf-8") as fh:
             raw = json.load(fh)
     else:
@@ -263,6 +265,73 @@ def serve_run(args, name):
             "prompt_tokens_computed": stats["num_prompt_tokens"], "dtype": args.dtype, "weights": "random"}
 
 
+# Layer sizes for --compare: (layers, width, heads), head size 128, a vocabulary of 32,768.
+COMPARE_SIZES = [(4, 1024, 8), (4, 2048, 16), (2, 4096, 32)]
+
+
+def viperax_like(layers, width, heads, vocab, window=512, streams=2):
+    """A Viperax config.json of a GPT-2-style model's size: the same layers, width, heads and
+    vocabulary; every token goes through 8 width^2 feed-forward elements a layer, as through the
+    GPT-2 MLP (dense layers with a hidden size of 8/3 width; every other layer 2 of 8 experts of
+    hidden size width beside a shared one of 2/3 width); latents of 128, read through a window;
+    the second half of the layers read the latents of the last layer of the first half."""
+    dim = width // heads
+    keep = layers // 2 - 1 if layers >= 4 else None
+    out = []
+    for i in range(layers):
+        mixer = {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": 128, "scale": dim ** -0.5, "mask": {"size": window}}
+        if keep is not None and i > keep:
+            mixer["kv_from"] = keep
+        if i % 2:
+            mlp = {"kind": "moe", "expert": {"ff": width}, "router": {"experts": 8, "top": 2},
+                   "shared": {"ff": width * 2 // 3 // 64 * 64}}
+        else:
+            mlp = {"kind": "dense", "ff": width * 8 // 3 // 64 * 64}
+        out.append({"type": "latent_attention", "mixer": mixer, "mlp": mlp})
+    return {"architecture": "Viperax", "vocab": vocab, "width": width, "streams": streams, "norm": {"eps": 1e-5},
+            "embedding": {"scale": float(width) ** 0.5}, "logit_scale": 1.0, "logit_softcap": 30.0, "layers": out}
+
+
+def compare_run(args, name):
+    """--compare viperax: prefill (2 prompts of 1,024 tokens as one step) and decode (batch 8, by the
+    default run's timing rule, fewer blocks) of Viperax beside the GPT-2-style model at equal layers,
+    width, heads and vocabulary, random weights, at COMPARE_SIZES.  One JSON line."""
+    import argparse as _argparse
+    import gc
+
+    import torch
+
+    assert name == "viperax"
+    vocab, rows = 32768, []
+    for layers, width, heads in COMPARE_SIZES:
+        row = {"layers": layers, "width": width, "heads": heads, "vocab": vocab}
+        for label, raw in (("gpt2-mini", {"architecture": "gpt2-mini", "n_layer": layers, "n_embd": width,
+                                          "n_head": heads, "vocab_size": vocab, "block_size": args.positions,
+                                          "bias": True, "layer_norm_eps": 1e-5}),
+                           ("viperax", viperax_like(layers, width, heads, vocab))):
+            a = _argparse.Namespace(**vars(args))
+            a.raw_config = raw
+            pre = prefill_run(a, args.dtype, reps=10, warmups=5)
+            run = decode_run(a, args.batch, args.steps, args.warmup, args.dtype, max(3, min(args.blocks, 6)))
+            med = quartiles(sorted(run["blocks"]))[1]
+            cost = run["engine"].model.cost()
+            itemsize = 2 if args.dtype == "bfloat16" else 4
+            step_s = med / args.steps
+            read = cost.step_read_bytes(args.batch, [run["mean_context"]] * args.batch, itemsize)
+            row[label] = {"prefill_tokens_per_s": pre["value"], "prefill_ms": pre["ms"], "prefill_mfma_frac": pre["frac"],
+                          "decode_tokens_per_s": round(args.batch * args.steps / med, 1),
+                          "decode_ms_per_step": round(step_s * 1e3, 4),
+                          "decode_hbm_frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 5),
+                          "kernels_per_step": kernels_per_step(run["engine"], args.batch)}
+            del run
+            gc.collect()
+            torch.cuda.empty_cache()
+        rows.append(row)
+        print(f"[bench] compared {row}", file=sys.stderr, flush=True)
+    return {"compare": "viperax beside gpt2-mini at equal layers, width, heads and vocabulary", "dtype": args.dtype,
+            "batch": args.batch, "prompt_len": args.prompt, "prefill": "2 x 1024 tokens, one step", "rows": rows}
+
+
 def host_cost_run(args):
     """What the host pays to launch one mixed step of the GPT-2-small shape (eight single tokens
     beside a prompt portion of 300, no HIP graph): through the model's Python, and from the plan
@@ -367,6 +436,8 @@ def main(argv=None) -> int:
                          "commit and the software and device that ran them")
     ap.add_argument("--prefill-requests", type=int, default=2,
                     help="prompts of 1,024 tokens in the prefill step (the contract's 2,048 tokens are 2)")
+    ap.add_argument("--compare", choices=["viperax"], default=None,
+                    help="prefill and decode of that design beside the GPT-2-style model at equal sizes (COMPARE_SIZES)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill and print its record (for profiling)")
     args = ap.parse_args(argv)
@@ -374,6 +445,9 @@ def main(argv=None) -> int:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
 
+    if args.compare:
+        print(json.dumps(compare_run(args, args.compare)))
+        return 0
     if args.prefill_only:
         print(json.dumps({"prefill": prefill_run(args, args.dtype)}))
         return 0

@@ -5,7 +5,7 @@
 //
 // experts: a token's id picks a row of `top` experts from an integer table.  A (token, choice)
 // pair is one unit of work.  The route kernel sorts the pairs by expert into slots; every expert's
-// run of slots is padded to a multiple of EX_TILE, so a tile of slots belongs to one expert
+// run of slots is padded to a multiple of the tile size (16 or 64 slots), so a tile of slots belongs to one expert
 // (tile_expert[tile], -1 for a tile that no expert uses) and slot_token[slot] is the pair's token
 // row (-1 for padding), slot_pair[slot] the pair's own index n * top + k.  The grouped product
 // then multiplies each tile by its expert's matrix; rows come from, and go to, the places that the
@@ -56,7 +56,7 @@ extern "C" int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int
 __global__ __launch_bounds__(256) void expert_route_kernel(
     const int* __restrict__ ids, const int* __restrict__ q_req, const int* __restrict__ table, int top,
     int n_rows, int n_experts, int* __restrict__ slot_token, int* __restrict__ slot_pair,
-    int* __restrict__ tile_expert, int n_slots, int n_tiles) {
+    int* __restrict__ tile_expert, int n_slots, int n_tiles, int tile_rows) {
   __shared__ int count[EX_MAX_EXPERTS];
   __shared__ int start[EX_MAX_EXPERTS];
   const int tid = threadIdx.x;
@@ -76,9 +76,9 @@ __global__ __launch_bounds__(256) void expert_route_kernel(
     int at = 0;
     for (int e = 0; e < n_experts; ++e) {
       start[e] = at;
-      const int tiles = (count[e] + EX_TILE - 1) / EX_TILE;
-      for (int t = 0; t < tiles; ++t) tile_expert[at / EX_TILE + t] = e;
-      at += tiles * EX_TILE;
+      const int tiles = (count[e] + tile_rows - 1) / tile_rows;
+      for (int t = 0; t < tiles; ++t) tile_expert[at / tile_rows + t] = e;
+      at += tiles * tile_rows;
       count[e] = 0;
     }
   }
@@ -94,20 +94,22 @@ __global__ __launch_bounds__(256) void expert_route_kernel(
   }
 }
 
-// n_slots >= n_rows * top + n_experts * (EX_TILE - 1) rounded up to whole tiles; n_tiles = n_slots / EX_TILE
+// tile_rows: 16 or 64 slots a tile; n_slots = n_tiles * tile_rows must hold n_rows * top pairs with
+// every used expert's run padded to whole tiles
 extern "C" int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows,
                                  int n_experts, int* slot_token, int* slot_pair, int* tile_expert, int n_slots,
-                                 int n_tiles, hipStream_t stream) {
+                                 int n_tiles, int tile_rows, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!ids || !table || !slot_token || !slot_pair || !tile_expert) return MGPT_ERR_NULL;
-  if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || n_slots != n_tiles * EX_TILE)
+  if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64) ||
+      n_slots != n_tiles * tile_rows)
     return MGPT_ERR_BAD_SHAPE;
   // every expert that is used wastes less than a tile
   const long pairs = (long)n_rows * top;
-  const long worst = pairs + (n_experts < pairs ? n_experts : pairs) * (long)(EX_TILE - 1);
-  if ((long)n_slots < worst / EX_TILE * EX_TILE) return MGPT_ERR_BAD_SHAPE;
+  const long worst = pairs + (n_experts < pairs ? n_experts : pairs) * (long)(tile_rows - 1);
+  if ((long)n_slots < worst / tile_rows * tile_rows) return MGPT_ERR_BAD_SHAPE;
   hipLaunchKernelGGL(expert_route_kernel, dim3(1), dim3(256), 0, stream, ids, q_req, table, top, n_rows, n_experts,
-                     slot_token, slot_pair, tile_expert, n_slots, n_tiles);
+                     slot_token, slot_pair, tile_expert, n_slots, n_tiles, tile_rows);
   return mgpt_last_error();
 }
 
@@ -115,11 +117,11 @@ template <typename T, typename OT>
 __global__ __launch_bounds__(256) void grouped_linear_kernel(
     const T* __restrict__ A, long lda, const int* __restrict__ a_rows, const T* __restrict__ W, long w_stride,
     const int* __restrict__ tile_expert, const int* __restrict__ slot_token, OT* __restrict__ out, long ldo,
-    const int* __restrict__ out_rows, int n_out, int k_dim) {
+    const int* __restrict__ out_rows, int n_out, int k_dim, int blocks_per_tile) {
   __shared__ float As[EX_TILE][EX_BK + 1];
   __shared__ float Ws[EX_TILE][EX_BK + 1];
-  const int tile = blockIdx.y;
-  const int e = tile_expert[tile];
+  const int tile = blockIdx.y;                    // 16 slots; blocks_per_tile of them share an expert
+  const int e = tile_expert[tile / blocks_per_tile];
   if (e < 0) return;
   const int tid = threadIdx.x;
   const int r = tid >> 4, c = tid & 15;
@@ -149,25 +151,116 @@ __global__ __launch_bounds__(256) void grouped_linear_kernel(
   out[orow * ldo + col] = from_float<OT>(acc);
 }
 
-// out[out_rows[s] or s] = A[a_rows[s] or s] @ W[tile_expert[s / EX_TILE]]^T for every slot s with
+// out[out_rows[s] or s] = A[a_rows[s] or s] @ W[tile_expert[s / tile_rows]]^T for every slot s with
 // slot_token[s] >= 0.  W: [experts][n_out][k_dim], w_stride elements from one expert to the next.
 extern "C" int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride,
                                    const int* tile_expert, const int* slot_token, void* out, int out_dtype,
-                                   long ldo, const int* out_rows, int n_tiles, int n_out, int k_dim, int dtype,
-                                   hipStream_t stream) {
+                                   long ldo, const int* out_rows, int n_tiles, int tile_rows, int n_out, int k_dim,
+                                   int dtype, hipStream_t stream) {
   if (n_tiles == 0 || n_out == 0) return MGPT_OK;
   if (!a || !w || !tile_expert || !slot_token || !out) return MGPT_ERR_NULL;
-  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out) return MGPT_ERR_BAD_SHAPE;
-  if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
-  dim3 grid((n_out + EX_TILE - 1) / EX_TILE, n_tiles), block(256);
+  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out || (tile_rows != 16 && tile_rows != 64))
+    return MGPT_ERR_BAD_SHAPE;
+  const int blocks_per_tile = tile_rows / EX_TILE;
+  if ((long)n_tiles * blocks_per_tile > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((n_out + EX_TILE - 1) / EX_TILE, n_tiles * blocks_per_tile), block(256);
 #define GL_LAUNCH(T, OT)                                                                                     \
   hipLaunchKernelGGL((grouped_linear_kernel<T, OT>), grid, block, 0, stream, (const T*)a, lda, a_rows,       \
-                     (const T*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows, n_out, k_dim)
+                     (const T*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows, n_out, k_dim,         \
+                     blocks_per_tile)
   if (dtype == MGPT_F32 && out_dtype == MGPT_F32) GL_LAUNCH(float, float);
   else if (dtype == MGPT_BF16 && out_dtype == MGPT_BF16) GL_LAUNCH(bf16_t, bf16_t);
   else if (dtype == MGPT_BF16 && out_dtype == MGPT_F32) GL_LAUNCH(bf16_t, float);
   else return MGPT_ERR_BAD_DTYPE;
 #undef GL_LAUNCH
+  return mgpt_last_error();
+}
+
+// The grouped product in bfloat16 on the MFMA units, for tiles of 64 slots.  A workgroup owns a
+// tile x 64 columns, a wave 16 of the columns for all 64 slots: per 32 k one slice of the expert's
+// matrix (first operand) and four slices of gathered rows, 16 bytes a lane straight from memory.
+typedef __attribute__((__vector_size__(8 * sizeof(short)))) short ex_bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ex_f32x4_t;
+
+template <typename OT>
+__global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
+    const bf16_t* __restrict__ A, long lda, const int* __restrict__ a_rows, const bf16_t* __restrict__ W,
+    long w_stride, const int* __restrict__ tile_expert, const int* __restrict__ slot_token, OT* __restrict__ out,
+    long ldo, const int* __restrict__ out_rows, int n_out, int k_dim) {
+  const int tile = blockIdx.y;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int col0 = blockIdx.x * 64 + wave * 16;
+  if (col0 >= n_out) return;
+  const int li = lane & 15, lg = lane >> 4;
+  const bool w_ok = col0 + li < n_out;
+  const bf16_t* wrow = W + (long)e * w_stride + (long)(w_ok ? col0 + li : 0) * k_dim;
+  const bf16_t* arow[4];
+  bool a_ok[4];
+  long orow[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int slot = tile * 64 + 16 * t + li;
+    a_ok[t] = slot_token[slot] >= 0;
+    arow[t] = A + (a_ok[t] ? (long)(a_rows ? a_rows[slot] : slot) : 0L) * lda;
+    orow[t] = a_ok[t] ? (long)(out_rows ? out_rows[slot] : slot) : 0L;
+  }
+  const ex_bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  ex_f32x4_t acc[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) acc[t] = ex_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < k_dim; k0 += 32) {
+    const int k = k0 + lg * 8;
+    const bool k_ok = k < k_dim;
+    const ex_bf16x8_t wf = (w_ok && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(wrow + k) : zero;
+    ex_bf16x8_t af[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      af[t] = (a_ok[t] && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(arow[t] + k) : zero;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af[t], acc[t], 0, 0, 0);
+  }
+  const int c = col0 + lg * 4;
+  if (c >= n_out) return;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    if (!a_ok[t]) continue;
+    OT* dst = out + orow[t] * ldo + c;
+    if (sizeof(OT) == 4) {
+      *reinterpret_cast<float4*>(dst) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+    } else {
+      uint2 pk;
+      pk.x = pack_bf16x2(acc[t][0], acc[t][1]);
+      pk.y = pack_bf16x2(acc[t][2], acc[t][3]);
+      *reinterpret_cast<uint2*>(dst) = pk;
+    }
+  }
+}
+
+// bfloat16 operands, tiles of 64 slots, bfloat16 or float32 out.  Refuses (MGPT_ERR_BAD_SHAPE) inner
+// sizes that are no multiple of 8, outputs that are no multiple of 4 and unaligned rows or bases;
+// the caller then takes mgpt_grouped_linear.
+extern "C" int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const void* w, long w_stride,
+                                        const int* tile_expert, const int* slot_token, void* out, int out_dtype,
+                                        long ldo, const int* out_rows, int n_tiles, int n_out, int k_dim,
+                                        hipStream_t stream) {
+  if (n_tiles == 0 || n_out == 0) return MGPT_OK;
+  if (!a || !w || !tile_expert || !slot_token || !out) return MGPT_ERR_NULL;
+  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out) return MGPT_ERR_BAD_SHAPE;
+  const int out_align = out_dtype == MGPT_F32 ? 15 : 7;
+  if ((k_dim & 7) || (n_out & 3) || (lda & 7) || (ldo & 3) || (w_stride & 7) || (((size_t)a | (size_t)w) & 15) ||
+      (((size_t)out) & out_align))
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
+  dim3 grid((n_out + 63) / 64, n_tiles), block(256);
+#define GM_LAUNCH(OT)                                                                                         \
+  hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT>), grid, block, 0, stream, (const bf16_t*)a, lda, a_rows, \
+                     (const bf16_t*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows, n_out, k_dim)
+  if (out_dtype == MGPT_F32) GM_LAUNCH(float);
+  else if (out_dtype == MGPT_BF16) GM_LAUNCH(bf16_t);
+  else return MGPT_ERR_BAD_DTYPE;
+#undef GM_LAUNCH
   return mgpt_last_error();
 }
 

@@ -124,14 +124,19 @@ int mgpt_rms_norm_store(const void* src, int dtype, long ld, const float* gain, 
     slot_mapping, int n_tokens, int rank, hipStream_t stream);
 int mgpt_heads_linear(const void* a, long lda, const void* w, void* out, long ldo, const void* gate, long ldg,
     int n_rows, int n_head, int n_out, int k_dim, int dtype, int fast, hipStream_t stream);
+int mgpt_heads_linear_mfma(const void* a, long lda, const void* w, void* out, long ldo, const void* gate, long ldg,
+    int n_rows, int n_head, int n_out, int k_dim, hipStream_t stream);
 // experts.hip
 int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype, int fast,
     hipStream_t stream);
 int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows, int n_experts,
-    int* slot_token, int* slot_pair, int* tile_expert, int n_slots, int n_tiles, hipStream_t stream);
+    int* slot_token, int* slot_pair, int* tile_expert, int n_slots, int n_tiles, int tile_rows, hipStream_t stream);
 int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
     tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
-    int n_out, int k_dim, int dtype, hipStream_t stream);
+    int tile_rows, int n_out, int k_dim, int dtype, hipStream_t stream);
+int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
+    tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
+    int n_out, int k_dim, hipStream_t stream);
 int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, int top, float weight,
     hipStream_t stream);
 }
@@ -168,6 +173,8 @@ int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, 
   X(mgpt_scale_softcap) \
   X(mgpt_rms_norm_store) \
   X(mgpt_heads_linear) \
+  X(mgpt_heads_linear_mfma) \
+  X(mgpt_grouped_linear_mfma) \
   X(mgpt_gated_unit) \
   X(mgpt_expert_route) \
   X(mgpt_grouped_linear) \

@@ -1029,6 +1029,14 @@ def heads_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_rows: in
     for name, t in (("out", out), ("gate", gate)):
         _need(t is None or (t.dim() == 2 and t.stride(1) == 1 and t.shape[1] >= n_head * n_out and t.shape[0] >= n_rows),
               f"{name} must be [>=n_rows, >=heads * out] with unit inner stride")
+    ldg = 0 if gate is None else gate.stride(0)
+    if fast and a.dtype == torch.bfloat16:
+        # the MFMA kernel; it refuses sizes and alignments that its 16-byte loads do not take
+        rc = library.kernels().mgpt_heads_linear_mfma(_ptr(a), a.stride(0), _ptr(w), _ptr(out), out.stride(0),
+                                                      _ptr(gate), ldg, n_rows, n_head, n_out, k_dim, _stream())
+        if rc != -2:
+            _check(rc, "heads_linear_mfma")
+            return
     rc = library.kernels().mgpt_heads_linear(_ptr(a), a.stride(0), _ptr(w), _ptr(out), out.stride(0), _ptr(gate),
                                              0 if gate is None else gate.stride(0), n_rows, n_head, n_out, k_dim,
                                              _dtype_code(a), int(fast), _stream())
@@ -1036,7 +1044,7 @@ def heads_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_rows: in
 
 
 # ---------------------------------------------------------------- gated feed-forwards and experts
-EXPERT_TILE = 16
+EXPERT_TILES = (16, 64)     # slots a tile: 16 for the general kernel, 64 for the MFMA kernel
 MAX_EXPERTS = 1024
 
 
@@ -1051,55 +1059,66 @@ def gated_unit(z: torch.Tensor, act: torch.Tensor, n_rows: int, hidden: int, fas
     _check(rc, "gated_unit")
 
 
-def expert_slots(n_rows: int, top: int, n_experts: int) -> int:
+def expert_slots(n_rows: int, top: int, n_experts: int, tile: int) -> int:
     """Slots that n_rows tokens with `top` experts each may need once every expert's run of slots is
-    padded to whole tiles."""
+    padded to whole tiles of `tile` slots."""
     pairs = n_rows * top
-    worst = pairs + min(n_experts, pairs) * (EXPERT_TILE - 1)
-    return -(-worst // EXPERT_TILE) * EXPERT_TILE
+    worst = pairs + min(n_experts, pairs) * (tile - 1)
+    return -(-worst // tile) * tile
 
 
 def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.Tensor, n_rows: int, n_experts: int,
-                 slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor) -> None:
+                 slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor, tile: int) -> None:
     """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip."""
     _need_cuda(ids, q_req, table, slot_token, slot_pair, tile_expert)
     _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "the table must be dense int32")
+    _need(tile in EXPERT_TILES, f"tiles of {EXPERT_TILES} slots")
     top = table.shape[1]
-    n_slots = expert_slots(n_rows, top, n_experts)
+    n_slots = expert_slots(n_rows, top, n_experts, tile)
     _need(n_experts <= MAX_EXPERTS, f"the route kernel takes up to {MAX_EXPERTS} experts")
     _need_i32("ids", ids, n_rows)
     if q_req is not None:
         _need_i32("q_req", q_req, n_rows)
     _need_i32("slot_token", slot_token, n_slots)
     _need_i32("slot_pair", slot_pair, n_slots)
-    _need_i32("tile_expert", tile_expert, n_slots // EXPERT_TILE)
+    _need_i32("tile_expert", tile_expert, n_slots // tile)
     rc = library.kernels().mgpt_expert_route(_ptr(ids), _ptr(q_req), _ptr(table), top, n_rows, n_experts,
                                              _ptr(slot_token), _ptr(slot_pair), _ptr(tile_expert), n_slots,
-                                             n_slots // EXPERT_TILE, _stream())
+                                             n_slots // tile, tile, _stream())
     _check(rc, "expert_route")
 
 
 def grouped_linear(a: torch.Tensor, a_rows: Optional[torch.Tensor], w: torch.Tensor, tile_expert: torch.Tensor,
-                   slot_token: torch.Tensor, out: torch.Tensor, out_rows: Optional[torch.Tensor], n_slots: int) -> None:
+                   slot_token: torch.Tensor, out: torch.Tensor, out_rows: Optional[torch.Tensor], n_slots: int,
+                   tile: int, fast: bool = False) -> None:
     """out[out_rows[s] or s] = a[a_rows[s] or s] @ w[expert of s's tile].T for every used slot s < n_slots.
     w: [experts, n_out, k_dim]."""
     _need_cuda(a, a_rows, w, tile_expert, slot_token, out, out_rows)
     _need(w.dim() == 3 and w.is_contiguous(), "the experts' matrices must be dense [experts, out, in]")
     _, n_out, k_dim = w.shape
-    _need(n_slots % EXPERT_TILE == 0, "slots come in whole tiles")
+    _need(tile in EXPERT_TILES and n_slots % tile == 0, "slots come in whole tiles")
     _need(a.dtype == w.dtype and a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim,
           "activations must be [rows, in] in the matrices' dtype")
     _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_out, "out must be [rows, out]")
     _need(a_rows is not None or a.shape[0] >= n_slots, "activations have fewer rows than slots")
     _need(out_rows is not None or out.shape[0] >= n_slots, "out has fewer rows than slots")
     _need_i32("slot_token", slot_token, n_slots)
-    _need_i32("tile_expert", tile_expert, n_slots // EXPERT_TILE)
+    _need_i32("tile_expert", tile_expert, n_slots // tile)
     for t in (a_rows, out_rows):
         if t is not None:
             _need_i32("row index", t, n_slots)
+    if fast and tile == 64 and a.dtype == torch.bfloat16:
+        # the MFMA kernel; it refuses sizes and alignments that its 16-byte loads do not take
+        rc = library.kernels().mgpt_grouped_linear_mfma(_ptr(a), a.stride(0), _ptr(a_rows), _ptr(w), w.stride(0),
+                                                        _ptr(tile_expert), _ptr(slot_token), _ptr(out),
+                                                        _dtype_code(out), out.stride(0), _ptr(out_rows),
+                                                        n_slots // tile, n_out, k_dim, _stream())
+        if rc != -2:
+            _check(rc, "grouped_linear_mfma")
+            return
     rc = library.kernels().mgpt_grouped_linear(_ptr(a), a.stride(0), _ptr(a_rows), _ptr(w), w.stride(0),
                                                _ptr(tile_expert), _ptr(slot_token), _ptr(out), _dtype_code(out),
-                                               out.stride(0), _ptr(out_rows), n_slots // EXPERT_TILE, n_out, k_dim,
+                                               out.stride(0), _ptr(out_rows), n_slots // tile, tile, n_out, k_dim,
                                                _dtype_code(a), _stream())
     _check(rc, "grouped_linear")
 

@@ -155,10 +155,12 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         # latent attention
         "mgpt_rms_norm_store": [P, I, L, P, F, P, P, I, I, P],
         "mgpt_heads_linear": [P, L, P, P, L, P, L, I, I, I, I, I, I, P],
+        "mgpt_heads_linear_mfma": [P, L, P, P, L, P, L, I, I, I, I, P],
         # gated feed-forwards and experts
         "mgpt_gated_unit": [P, L, P, L, I, I, I, I, P],
-        "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, I, I, P],
-        "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, P],
+        "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, I, I, I, P],
+        "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, I, P],
+        "mgpt_grouped_linear_mfma": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, P],
         "mgpt_expert_combine": [P, P, I, I, I, F, P],
     }
     for name, argtypes in table.items():

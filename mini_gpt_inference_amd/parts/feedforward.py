@@ -190,17 +190,22 @@ class TableExperts(FeedForward):
         plain_residual(ctx, h, x)
         n, ws = ctx.n_rows, ctx.workspace
         hn = as_tensor(ctx, h)
-        slots = kernels.expert_slots(n, self.top, self.n_experts)
+        # tiles of 64 slots for the MFMA kernel, of 16 for the general one
+        fast = not ctx.exact and ctx.dtype == torch.bfloat16
+        tile = 64 if fast else 16
+        slots = kernels.expert_slots(n, self.top, self.n_experts, tile)
         slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
         slot_pair = ws.get("expert_slot_pair", slots, 1, torch.int32).view(-1)
-        tile_expert = ws.get("expert_tile", slots // kernels.EXPERT_TILE, 1, torch.int32).view(-1)
-        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair, tile_expert)
+        tile_expert = ws.get("expert_tile", slots // tile, 1, torch.int32).view(-1)
+        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair,
+                             tile_expert, tile)
         z = ws.get("expert_z", slots, 2 * self.hidden, ctx.dtype)
-        kernels.grouped_linear(hn, slot_token, self.in_weights, tile_expert, slot_token, z, None, slots)
+        kernels.grouped_linear(hn, slot_token, self.in_weights, tile_expert, slot_token, z, None, slots, tile, fast)
         act = ws.get("expert_act", slots, self.hidden, ctx.dtype)
         kernels.gated_unit(z, act, slots, self.hidden, fast=not ctx.exact)
         pair_out = ws.get("expert_pair_out", n * self.top, self.width, torch.float32)
-        kernels.grouped_linear(act, None, self.down_weights, tile_expert, slot_token, pair_out, slot_pair, slots)
+        kernels.grouped_linear(act, None, self.down_weights, tile_expert, slot_token, pair_out, slot_pair, slots,
+                               tile, fast)
         if self.shared_hidden:
             _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
         kernels.expert_combine(pair_out, x, n, self.top, 1.0 / self.top)

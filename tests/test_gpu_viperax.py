@@ -96,7 +96,8 @@ def test_rms_norm_store(dtype, rank, page):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,heads,n_out,k", [(1, 1, 40, 24), (19, 3, 16, 96), (70, 4, 96, 64), (5, 2, 7, 130)])
+@pytest.mark.parametrize("n,heads,n_out,k", [(1, 1, 40, 24), (19, 3, 16, 96), (70, 4, 96, 64), (5, 2, 7, 130),
+                                             (200, 5, 72, 40), (65, 2, 128, 128)])
 def test_heads_linear_with_and_without_gate(dtype, n, heads, n_out, k):
     g = torch.Generator().manual_seed(n)
     a = _rnd(g, n, heads * k + 8, dtype=dtype)
@@ -119,10 +120,11 @@ def test_gated_unit(dtype):
     helpers.assert_close(act, V.silu(z[:, :37].float()) * z[:, 37:].float(), dtype, "gated unit")
 
 
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("dtype,tile,fast", [("float32", 16, False), ("bfloat16", 16, False), ("bfloat16", 64, True),
+                                             ("float32", 64, False)])
 @pytest.mark.parametrize("n,experts,top,width,hidden", [(1, 2, 1, 24, 8), (40, 5, 2, 64, 24), (300, 16, 1, 48, 40),
-                                                        (7, 3, 3, 32, 16)])
-def test_experts_by_table(dtype, n, experts, top, width, hidden):
+                                                        (7, 3, 3, 32, 16), (130, 4, 2, 100, 36)])
+def test_experts_by_table(dtype, tile, fast, n, experts, top, width, hidden):
     """Route, both grouped products, the gated unit and the sum over a token's experts, against the
     plain loop; some tokens are padding (their request is -1) and an expert may get no token."""
     g = torch.Generator().manual_seed(n)
@@ -137,22 +139,22 @@ def test_experts_by_table(dtype, n, experts, top, width, hidden):
     h = _rnd(g, n, width, dtype=dtype)
     w_in = _rnd(g, experts, 2 * hidden, width, dtype=dtype, scale=width ** -0.5)
     w_down = _rnd(g, experts, width, hidden, dtype=dtype, scale=hidden ** -0.5)
-    slots = kernels.expert_slots(n, top, experts)
+    slots = kernels.expert_slots(n, top, experts, tile)
     st, sp = (torch.full((slots,), -7, dtype=torch.int32, device=DEV) for _ in range(2))
-    te = torch.full((slots // kernels.EXPERT_TILE,), -7, dtype=torch.int32, device=DEV)
-    kernels.expert_route(ids.to(DEV), q_req.to(DEV), table.to(DEV), n, experts, st, sp, te)
+    te = torch.full((slots // tile,), -7, dtype=torch.int32, device=DEV)
+    kernels.expert_route(ids.to(DEV), q_req.to(DEV), table.to(DEV), n, experts, st, sp, te, tile)
     z = torch.zeros(slots, 2 * hidden, dtype=TDT[dtype], device=DEV)
-    kernels.grouped_linear(h.to(DEV), st, w_in.to(DEV), te, st, z, None, slots)
+    kernels.grouped_linear(h.to(DEV), st, w_in.to(DEV), te, st, z, None, slots, tile, fast)
     act = torch.zeros(slots, hidden, dtype=TDT[dtype], device=DEV)
     kernels.gated_unit(z, act, slots, hidden, fast=dtype == "bfloat16")
     pair_out = torch.zeros(n * top, width, device=DEV)
-    kernels.grouped_linear(act, None, w_down.to(DEV), te, st, pair_out, sp, slots)
+    kernels.grouped_linear(act, None, w_down.to(DEV), te, st, pair_out, sp, slots, tile, fast)
     y = torch.ones(n, width, device=DEV)
     kernels.expert_combine(pair_out, y, n, top, 1.0 / top)
     live = [i for i in range(n) if q_req[i] >= 0]
     # every live pair has exactly one slot, in a tile of its expert
     st_h, sp_h, te_h = st.cpu(), sp.cpu(), te.cpu()
-    used = [(int(sp_h[s]), int(te_h[s // kernels.EXPERT_TILE])) for s in range(slots) if st_h[s] >= 0]
+    used = [(int(sp_h[s]), int(te_h[s // tile])) for s in range(slots) if st_h[s] >= 0]
     assert sorted(p for p, _ in used) == sorted(i * top + j for i in live for j in range(top))
     assert all(e == int(table[ids[p // top], p % top]) for p, e in used)
     exp = [(w_in[e, :hidden].float(), w_in[e, hidden:].float(), w_down[e].float()) for e in range(experts)]
