@@ -311,6 +311,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) o[dt][i] = o[dt][i] * a0 + xch[2 + dt * 4 + i] * a1;
+    m = m_all;   // what the sums are relative to from here on (a sink joins them below)
   }
 
   l = pf_sum_over_rows(l);

@@ -51,12 +51,40 @@ extern "C" int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int
   return mgpt_last_error();
 }
 
+// sorted[s] = src[slot_token[s]] for every used slot: the rows of a step in the experts' order, 16 bytes a lane
+__global__ void gather_rows_kernel(const uint4* __restrict__ src, long ld16, const int* __restrict__ slot_token,
+                                   uint4* __restrict__ sorted, long lds16, int n_slots, int chunks) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= (long)n_slots * chunks) return;
+  const long s = i / chunks;
+  const int c = (int)(i - s * chunks);
+  const int row = slot_token[s];
+  if (row < 0) return;
+  sorted[s * lds16 + c] = src[row * ld16 + c];
+}
+
+// bfloat16 rows of `width` (a multiple of 8) elements, 16-byte aligned
+extern "C" int mgpt_gather_rows(const void* src, long ld, const int* slot_token, void* sorted, long lds, int n_slots,
+                                int width, hipStream_t stream) {
+  if (n_slots == 0) return MGPT_OK;
+  if (!src || !slot_token || !sorted) return MGPT_ERR_NULL;
+  if (n_slots < 0 || width <= 0 || (width & 7) || (ld & 7) || (lds & 7) || ld < width || lds < width ||
+      (((size_t)src | (size_t)sorted) & 15))
+    return MGPT_ERR_BAD_SHAPE;
+  const long total = (long)n_slots * (width / 8);
+  const long blocks = (total + 255) / 256;
+  if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(gather_rows_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const uint4*)src, ld / 8,
+                     slot_token, (uint4*)sorted, lds / 8, n_slots, width / 8);
+  return mgpt_last_error();
+}
+
 // One workgroup: counts the pairs of every expert, lays the experts' runs of slots out one after
 // the other (each padded to whole tiles), and deals the pairs into them.
-__global__ __launch_bounds__(256) void expert_route_kernel(
+__global__ __launch_bounds__(1024) void expert_route_kernel(
     const int* __restrict__ ids, const int* __restrict__ q_req, const int* __restrict__ table, int top,
     int n_rows, int n_experts, int* __restrict__ slot_token, int* __restrict__ slot_pair,
-    int* __restrict__ tile_expert, int n_slots, int n_tiles, int tile_rows) {
+    int* __restrict__ pair_slot, int* __restrict__ tile_expert, int n_slots, int n_tiles, int tile_rows) {
   __shared__ int count[EX_MAX_EXPERTS];
   __shared__ int start[EX_MAX_EXPERTS];
   const int tid = threadIdx.x;
@@ -91,25 +119,26 @@ __global__ __launch_bounds__(256) void expert_route_kernel(
     const int s = start[e] + atomicAdd(&count[e], 1);
     slot_token[s] = n;
     slot_pair[s] = p;
+    if (pair_slot) pair_slot[p] = s;
   }
 }
 
-// tile_rows: 16 or 64 slots a tile; n_slots = n_tiles * tile_rows must hold n_rows * top pairs with
-// every used expert's run padded to whole tiles
+// tile_rows: 16, 64 or 256 slots a tile; n_slots = n_tiles * tile_rows must hold n_rows * top pairs with
+// every used expert's run padded to whole tiles.  pair_slot (optional, [n_rows * top]): where each pair went.
 extern "C" int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows,
-                                 int n_experts, int* slot_token, int* slot_pair, int* tile_expert, int n_slots,
-                                 int n_tiles, int tile_rows, hipStream_t stream) {
+                                 int n_experts, int* slot_token, int* slot_pair, int* pair_slot, int* tile_expert,
+                                 int n_slots, int n_tiles, int tile_rows, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!ids || !table || !slot_token || !slot_pair || !tile_expert) return MGPT_ERR_NULL;
-  if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64) ||
-      n_slots != n_tiles * tile_rows)
+  if (n_rows < 0 || top <= 0 || n_experts <= 0 || n_experts > EX_MAX_EXPERTS || (tile_rows != 16 && tile_rows != 64 && tile_rows != 256) || n_slots != n_tiles * tile_rows)
     return MGPT_ERR_BAD_SHAPE;
   // every expert that is used wastes less than a tile
   const long pairs = (long)n_rows * top;
   const long worst = pairs + (n_experts < pairs ? n_experts : pairs) * (long)(tile_rows - 1);
   if ((long)n_slots < worst / tile_rows * tile_rows) return MGPT_ERR_BAD_SHAPE;
-  hipLaunchKernelGGL(expert_route_kernel, dim3(1), dim3(256), 0, stream, ids, q_req, table, top, n_rows, n_experts,
-                     slot_token, slot_pair, tile_expert, n_slots, n_tiles, tile_rows);
+  const int threads = (long)n_rows * top > 256 ? 1024 : 256;
+  hipLaunchKernelGGL(expert_route_kernel, dim3(1), dim3(threads), 0, stream, ids, q_req, table, top, n_rows, n_experts,
+                     slot_token, slot_pair, pair_slot, tile_expert, n_slots, n_tiles, tile_rows);
   return mgpt_last_error();
 }
 
@@ -159,7 +188,7 @@ extern "C" int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, c
                                    int dtype, hipStream_t stream) {
   if (n_tiles == 0 || n_out == 0) return MGPT_OK;
   if (!a || !w || !tile_expert || !slot_token || !out) return MGPT_ERR_NULL;
-  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out || (tile_rows != 16 && tile_rows != 64))
+  if (n_tiles < 0 || n_out < 0 || k_dim <= 0 || lda < k_dim || ldo < n_out || (tile_rows != 16 && tile_rows != 64 && tile_rows != 256))
     return MGPT_ERR_BAD_SHAPE;
   const int blocks_per_tile = tile_rows / EX_TILE;
   if ((long)n_tiles * blocks_per_tile > 65535) return MGPT_ERR_TOO_LARGE;
@@ -177,25 +206,33 @@ extern "C" int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, c
 }
 
 // The grouped product in bfloat16 on the MFMA units, for tiles of 64 slots.  A workgroup owns a
-// tile x 64 columns, a wave 16 of the columns for all 64 slots: per 32 k one slice of the expert's
-// matrix (first operand) and four slices of gathered rows, 16 bytes a lane straight from memory.
+// tile x 64 (or 256) columns, a wave 16 (or 64) of the columns for all 64 slots: per 32 k one (or four)
+// slices of the expert's matrix (first operand) and four slices of gathered rows, 16 bytes a lane
+// straight from memory.
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short ex_bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float ex_f32x4_t;
 
-template <typename OT>
+template <typename OT, int NJ>
 __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
     const bf16_t* __restrict__ A, long lda, const int* __restrict__ a_rows, const bf16_t* __restrict__ W,
     long w_stride, const int* __restrict__ tile_expert, const int* __restrict__ slot_token, OT* __restrict__ out,
     long ldo, const int* __restrict__ out_rows, int n_out, int k_dim) {
+  // a wave owns 64 slots x NJ * 16 columns: per 32 k it loads NJ slices of the matrix and four of the
+  // rows for 4 * NJ MFMAs
   const int tile = blockIdx.y;
   const int e = tile_expert[tile];
   if (e < 0) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int col0 = blockIdx.x * 64 + wave * 16;
+  const int col0 = (blockIdx.x * 4 + wave) * (NJ * 16);
   if (col0 >= n_out) return;
   const int li = lane & 15, lg = lane >> 4;
-  const bool w_ok = col0 + li < n_out;
-  const bf16_t* wrow = W + (long)e * w_stride + (long)(w_ok ? col0 + li : 0) * k_dim;
+  const bf16_t* wrow[NJ];
+  bool w_ok[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    w_ok[j] = col0 + j * 16 + li < n_out;
+    wrow[j] = W + (long)e * w_stride + (long)(w_ok[j] ? col0 + j * 16 + li : 0) * k_dim;
+  }
   const bf16_t* arow[4];
   bool a_ok[4];
   long orow[4];
@@ -207,33 +244,43 @@ __global__ __launch_bounds__(256) void grouped_linear_mfma_kernel(
     orow[t] = a_ok[t] ? (long)(out_rows ? out_rows[slot] : slot) : 0L;
   }
   const ex_bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  ex_f32x4_t acc[4];
+  ex_f32x4_t acc[NJ][4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) acc[t] = ex_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NJ; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[j][t] = ex_f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < k_dim; k0 += 32) {
     const int k = k0 + lg * 8;
     const bool k_ok = k < k_dim;
-    const ex_bf16x8_t wf = (w_ok && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(wrow + k) : zero;
-    ex_bf16x8_t af[4];
+    ex_bf16x8_t wf[NJ], af[4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      wf[j] = (w_ok[j] && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(wrow[j] + k) : zero;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
       af[t] = (a_ok[t] && k_ok) ? *reinterpret_cast<const ex_bf16x8_t*>(arow[t] + k) : zero;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af[t], acc[t], 0, 0, 0);
-  }
-  const int c = col0 + lg * 4;
-  if (c >= n_out) return;
+    for (int j = 0; j < NJ; ++j)
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    if (!a_ok[t]) continue;
-    OT* dst = out + orow[t] * ldo + c;
-    if (sizeof(OT) == 4) {
-      *reinterpret_cast<float4*>(dst) = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-    } else {
-      uint2 pk;
-      pk.x = pack_bf16x2(acc[t][0], acc[t][1]);
-      pk.y = pack_bf16x2(acc[t][2], acc[t][3]);
-      *reinterpret_cast<uint2*>(dst) = pk;
+      for (int t = 0; t < 4; ++t)
+        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[t], acc[j][t], 0, 0, 0);
+  }
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    const int c = col0 + j * 16 + lg * 4;
+    if (c >= n_out) continue;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      if (!a_ok[t]) continue;
+      OT* dst = out + orow[t] * ldo + c;
+      if (sizeof(OT) == 4) {
+        *reinterpret_cast<float4*>(dst) = make_float4(acc[j][t][0], acc[j][t][1], acc[j][t][2], acc[j][t][3]);
+      } else {
+        uint2 pk;
+        pk.x = pack_bf16x2(acc[j][t][0], acc[j][t][1]);
+        pk.y = pack_bf16x2(acc[j][t][2], acc[j][t][3]);
+        *reinterpret_cast<uint2*>(dst) = pk;
+      }
     }
   }
 }
@@ -253,38 +300,46 @@ extern "C" int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_ro
       (((size_t)out) & out_align))
     return MGPT_ERR_BAD_SHAPE;
   if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
-  dim3 grid((n_out + 63) / 64, n_tiles), block(256);
-#define GM_LAUNCH(OT)                                                                                         \
-  hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT>), grid, block, 0, stream, (const bf16_t*)a, lda, a_rows, \
-                     (const bf16_t*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows, n_out, k_dim)
-  if (out_dtype == MGPT_F32) GM_LAUNCH(float);
-  else if (out_dtype == MGPT_BF16) GM_LAUNCH(bf16_t);
+  // wide outputs: a wave takes 64 columns; narrow ones 16, so that a tile still gives several workgroups
+  const bool wide = n_out >= 512;
+  dim3 grid((n_out + (wide ? 255 : 63)) / (wide ? 256 : 64), n_tiles), block(256);
+#define GM_LAUNCH(OT, NJ)                                                                                     \
+  hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT, NJ>), grid, block, 0, stream, (const bf16_t*)a, lda,     \
+                     a_rows, (const bf16_t*)w, w_stride, tile_expert, slot_token, (OT*)out, ldo, out_rows,    \
+                     n_out, k_dim)
+  if (out_dtype == MGPT_F32) { if (wide) GM_LAUNCH(float, 4); else GM_LAUNCH(float, 1); }
+  else if (out_dtype == MGPT_BF16) { if (wide) GM_LAUNCH(bf16_t, 4); else GM_LAUNCH(bf16_t, 1); }
   else return MGPT_ERR_BAD_DTYPE;
 #undef GM_LAUNCH
   return mgpt_last_error();
 }
 
-__global__ void expert_combine_kernel(const float* __restrict__ pair_out, float* __restrict__ y, long total,
-                                      int width, int top, float weight) {
+__global__ void expert_combine_kernel(const float* __restrict__ pair_out, const int* __restrict__ pair_slot,
+                                      const int* __restrict__ q_req, float* __restrict__ y, long total, int width,
+                                      int top, float weight) {
   const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
   if (i >= total) return;
   const long n = i / width;
   const int c = (int)(i - n * width);
+  if (q_req && q_req[n] < 0) return;   // padded token: its pairs went nowhere
   float acc = 0.f;
-  for (int k = 0; k < top; ++k) acc += pair_out[(n * top + k) * (long)width + c];
+  for (int k = 0; k < top; ++k) {
+    const long row = pair_slot ? pair_slot[n * top + k] : n * top + k;
+    acc += pair_out[row * (long)width + c];
+  }
   y[i] += acc * weight;
 }
 
-// y[n] += weight * sum_k pair_out[n * top + k]
-extern "C" int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, int top, float weight,
-                                   hipStream_t stream) {
+// y[n] += weight * sum_k pair_out[pair_slot[n * top + k]] (pair_slot null: row n * top + k itself)
+extern "C" int mgpt_expert_combine(const float* pair_out, const int* pair_slot, const int* q_req, float* y, int n_rows,
+                                   int width, int top, float weight, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!pair_out || !y) return MGPT_ERR_NULL;
   if (n_rows < 0 || width <= 0 || top <= 0) return MGPT_ERR_BAD_SHAPE;
   const long total = (long)n_rows * width;
   const long blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(expert_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, pair_out, y, total, width,
-                     top, weight);
+  hipLaunchKernelGGL(expert_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, pair_out, pair_slot, q_req, y,
+                     total, width, top, weight);
   return mgpt_last_error();
 }

@@ -130,14 +130,21 @@ int mgpt_heads_linear_mfma(const void* a, long lda, const void* w, void* out, lo
 int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype, int fast,
     hipStream_t stream);
 int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows, int n_experts,
-    int* slot_token, int* slot_pair, int* tile_expert, int n_slots, int n_tiles, int tile_rows, hipStream_t stream);
+    int* slot_token, int* slot_pair, int* pair_slot, int* tile_expert, int n_slots, int n_tiles, int tile_rows,
+    hipStream_t stream);
+int mgpt_gather_rows(const void* src, long ld, const int* slot_token, void* sorted, long lds, int n_slots, int width,
+    hipStream_t stream);
 int mgpt_grouped_linear(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
     tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
     int tile_rows, int n_out, int k_dim, int dtype, hipStream_t stream);
 int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const void* w, long w_stride, const int*
     tile_expert, const int* slot_token, void* out, int out_dtype, long ldo, const int* out_rows, int n_tiles,
     int n_out, int k_dim, hipStream_t stream);
-int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, int top, float weight,
+int mgpt_expert_combine(const float* pair_out, const int* pair_slot, const int* q_req, float* y, int n_rows, int
+    width, int top, float weight, hipStream_t stream);
+// linear_mfma.hip
+int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_stride, const int* row_expert, const
+    int* row_valid, int group_rows, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
     hipStream_t stream);
 }
 
@@ -178,4 +185,6 @@ int mgpt_expert_combine(const float* pair_out, float* y, int n_rows, int width, 
   X(mgpt_gated_unit) \
   X(mgpt_expert_route) \
   X(mgpt_grouped_linear) \
-  X(mgpt_expert_combine)
+  X(mgpt_expert_combine) \
+  X(mgpt_gather_rows) \
+  X(mgpt_linear_mfma_grouped)

@@ -48,6 +48,13 @@ struct MfmaScatter {
   bf16_t* vpool;
   const int* slot_mapping;  // per row: page * page_size + offset, or -1 for a padded row
   int q_width, kv_width, head_dim, n_kv_head, page_size;
+  // Rows in groups that each multiply a matrix of their own (experts): row r belongs to group
+  // r / group_rows, whose matrix is w + row_expert[group] * w_stride (a negative entry: the group is
+  // not in use); row_valid[r] < 0 marks padding at the end of a group.  Null: one matrix for all rows.
+  const int* row_expert = nullptr;
+  const int* row_valid = nullptr;
+  int group_rows = 0;
+  long w_stride = 0;
 };
 
 // The bias of the four neighbouring output columns oc..oc+3 a lane holds.
@@ -174,6 +181,12 @@ __global__ __launch_bounds__(64 * WVM * WVN * KG) void linear_mfma_kernel(
     col_tile = in_group / rows_here;
   }
   const int row0 = row_tile * BM, col0 = col_tile * BN;
+  if (sc.row_expert) {
+    // (the launcher has seen to it that a tile's rows lie in one group; padding comes last in a group)
+    const int e = sc.row_expert[row0 / sc.group_rows];
+    if (e < 0 || sc.row_valid[row0] < 0) return;   // the whole workgroup, before any barrier
+    w += (long)e * sc.w_stride;
+  }
   // this workgroup's stretch of the inner size (all of it unless the product is split), in whole steps
   const int k_per = (((k_dim + MM_BK - 1) / MM_BK + k_parts - 1) / k_parts) * MM_BK;
   const int k_begin = part * k_per;
@@ -919,6 +932,26 @@ extern "C" int mgpt_linear_mfma_shape(int shape, int k_parts, const void* act, l
   MfmaScatter sc = {};
   return launch_any(shape, k_parts, act, lda, w, bias, out, out_dtype, ldo, n_rows, n_out, k_dim, epilogue,
                     partials, partials_floats, sc, stream);
+}
+
+// Rows in groups of group_rows (256) that each multiply a matrix of their own: out[r] = act[r] W_e^T with
+// e = row_expert[r / group_rows] (negative: nothing is computed for the group) and W_e = w + e * w_stride;
+// row_valid[r] < 0 marks the padding that ends a group, and a tile that starts in it is skipped.  bfloat16 or
+// float32 out, no bias, the inner size never split.
+extern "C" int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_stride, const int* row_expert,
+                                        const int* row_valid, int group_rows, void* out, int out_dtype, long ldo,
+                                        int n_rows, int n_out, int k_dim, hipStream_t stream) {
+  if (!row_expert || !row_valid) return MGPT_ERR_NULL;
+  // every tile shape's rows (32 to 256) divide a group
+  if (group_rows != 256 || (n_rows % group_rows) != 0 || w_stride < (long)n_out * k_dim || (w_stride & 7) != 0)
+    return MGPT_ERR_BAD_SHAPE;
+  MfmaScatter sc = {};
+  sc.row_expert = row_expert;
+  sc.row_valid = row_valid;
+  sc.group_rows = group_rows;
+  sc.w_stride = w_stride;
+  return launch_any(-1, 1, act, lda, w, nullptr, out, out_dtype, ldo, n_rows, n_out, k_dim, MM_EPI_NONE, nullptr, 0, sc,
+                    stream);
 }
 
 // The fused QKV product of a step with prompt portions: out[n] = act[n] W^T + bias in bfloat16, and

@@ -1044,7 +1044,8 @@ def heads_linear(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, n_rows: in
 
 
 # ---------------------------------------------------------------- gated feed-forwards and experts
-EXPERT_TILES = (16, 64)     # slots a tile: 16 for the general kernel, 64 for the MFMA kernel
+# slots a tile: 16 for the general kernel, 64 for the MFMA kernel of few rows, 256 for the tiled MFMA kernel
+EXPERT_TILES = (16, 64, 256)
 MAX_EXPERTS = 1024
 
 
@@ -1068,9 +1069,11 @@ def expert_slots(n_rows: int, top: int, n_experts: int, tile: int) -> int:
 
 
 def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.Tensor, n_rows: int, n_experts: int,
-                 slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor, tile: int) -> None:
-    """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip."""
-    _need_cuda(ids, q_req, table, slot_token, slot_pair, tile_expert)
+                 slot_token: torch.Tensor, slot_pair: torch.Tensor, tile_expert: torch.Tensor, tile: int,
+                 pair_slot: Optional[torch.Tensor] = None) -> None:
+    """Sorts the (token, choice) pairs by expert into slots; see csrc/hip/experts.hip.  pair_slot
+    ([n_rows * top], optional) receives the slot of every pair."""
+    _need_cuda(ids, q_req, table, slot_token, slot_pair, tile_expert, pair_slot)
     _need(table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous(), "the table must be dense int32")
     _need(tile in EXPERT_TILES, f"tiles of {EXPERT_TILES} slots")
     top = table.shape[1]
@@ -1082,9 +1085,11 @@ def expert_route(ids: torch.Tensor, q_req: Optional[torch.Tensor], table: torch.
     _need_i32("slot_token", slot_token, n_slots)
     _need_i32("slot_pair", slot_pair, n_slots)
     _need_i32("tile_expert", tile_expert, n_slots // tile)
+    if pair_slot is not None:
+        _need_i32("pair_slot", pair_slot, n_rows * top)
     rc = library.kernels().mgpt_expert_route(_ptr(ids), _ptr(q_req), _ptr(table), top, n_rows, n_experts,
-                                             _ptr(slot_token), _ptr(slot_pair), _ptr(tile_expert), n_slots,
-                                             n_slots // tile, tile, _stream())
+                                             _ptr(slot_token), _ptr(slot_pair), _ptr(pair_slot), _ptr(tile_expert),
+                                             n_slots, n_slots // tile, tile, _stream())
     _check(rc, "expert_route")
 
 
@@ -1123,11 +1128,62 @@ def grouped_linear(a: torch.Tensor, a_rows: Optional[torch.Tensor], w: torch.Ten
     _check(rc, "grouped_linear")
 
 
-def expert_combine(pair_out: torch.Tensor, y: torch.Tensor, n_rows: int, top: int, weight: float) -> None:
-    """y[n] += weight * sum_k pair_out[n * top + k]; both float32."""
-    _need_cuda(pair_out, y)
+def expert_combine(pair_out: torch.Tensor, y: torch.Tensor, n_rows: int, top: int, weight: float,
+                   pair_slot: Optional[torch.Tensor] = None, q_req: Optional[torch.Tensor] = None) -> None:
+    """y[n] += weight * sum_k pair_out[pair_slot[n * top + k]] (without pair_slot: row n * top + k); both
+    float32.  Tokens whose q_req is negative (padding) are left alone."""
+    _need_cuda(pair_out, y, pair_slot, q_req)
     width = y.shape[1]
     _need_rows_f32("y", y, n_rows, width)
-    _need_rows_f32("pair_out", pair_out, n_rows * top, width)
-    rc = library.kernels().mgpt_expert_combine(_ptr(pair_out), _ptr(y), n_rows, width, top, float(weight), _stream())
+    if pair_slot is None:
+        _need_rows_f32("pair_out", pair_out, n_rows * top, width)
+    else:
+        _need_rows_f32("pair_out", pair_out, 0, width)      # its rows are slots: the route kernel's bound holds
+        _need_i32("pair_slot", pair_slot, n_rows * top)
+    if q_req is not None:
+        _need_i32("q_req", q_req, n_rows)
+    rc = library.kernels().mgpt_expert_combine(_ptr(pair_out), _ptr(pair_slot), _ptr(q_req), _ptr(y), n_rows, width,
+                                               top, float(weight), _stream())
     _check(rc, "expert_combine")
+
+
+def gather_rows(src: torch.Tensor, slot_token: torch.Tensor, out: torch.Tensor, n_slots: int) -> bool:
+    """out[s] = src[slot_token[s]] for every used slot s < n_slots (bfloat16 rows whose width is a
+    multiple of 8).  False, with nothing launched, for other rows."""
+    _need_cuda(src, slot_token, out)
+    width = src.shape[1]
+    if src.dtype != torch.bfloat16 or width % 8 or src.stride(0) % 8 or out.stride(0) % 8 \
+            or src.data_ptr() % 16 or out.data_ptr() % 16:
+        return False
+    _need(out.dtype == src.dtype and out.dim() == 2 and out.shape[1] == width and out.shape[0] >= n_slots
+          and src.stride(1) == 1 and out.stride(1) == 1, "out must be [>=n_slots, width] like src")
+    _need_i32("slot_token", slot_token, n_slots)
+    rc = library.kernels().mgpt_gather_rows(_ptr(src), src.stride(0), _ptr(slot_token), _ptr(out), out.stride(0),
+                                            n_slots, width, _stream())
+    _check(rc, "gather_rows")
+    return True
+
+
+def grouped_linear_tiled(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Tensor, slot_token: torch.Tensor,
+                         out: torch.Tensor, n_slots: int) -> bool:
+    """out[s] = a[s] @ w[expert of s's tile of 256].T for the slots of every tile in use, through the
+    tiled MFMA kernel (bfloat16 operands, bfloat16 or float32 out).  False, with nothing launched,
+    if that kernel does not take the sizes."""
+    _need_cuda(a, w, tile_expert, slot_token, out)
+    _need(w.dim() == 3 and w.is_contiguous(), "the experts' matrices must be dense [experts, out, in]")
+    _, n_out, k_dim = w.shape
+    if a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or k_dim % 16 or a.stride(0) % 8 or n_slots % 256:
+        return False
+    _need(a.dim() == 2 and a.stride(1) == 1 and a.shape[1] == k_dim and a.shape[0] >= n_slots,
+          "activations must be [>=n_slots, in]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] == n_out and out.shape[0] >= n_slots,
+          "out must be [>=n_slots, out]")
+    _need_i32("slot_token", slot_token, n_slots)
+    _need_i32("tile_expert", tile_expert, n_slots // 256)
+    rc = library.kernels().mgpt_linear_mfma_grouped(_ptr(a), a.stride(0), _ptr(w), w.stride(0), _ptr(tile_expert),
+                                                    _ptr(slot_token), 256, _ptr(out), _dtype_code(out), out.stride(0),
+                                                    n_slots, n_out, k_dim, _stream())
+    if rc == -2:
+        return False
+    _check(rc, "linear_mfma_grouped")
+    return True

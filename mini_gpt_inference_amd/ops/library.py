@@ -158,10 +158,12 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_heads_linear_mfma": [P, L, P, P, L, P, L, I, I, I, I, P],
         # gated feed-forwards and experts
         "mgpt_gated_unit": [P, L, P, L, I, I, I, I, P],
-        "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, I, I, I, P],
+        "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, P, I, I, I, P],
+        "mgpt_gather_rows": [P, L, P, P, L, I, I, P],
+        "mgpt_linear_mfma_grouped": [P, L, P, L, P, P, I, P, I, L, I, I, I, P],
         "mgpt_grouped_linear": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, I, I, P],
         "mgpt_grouped_linear_mfma": [P, L, P, P, L, P, P, P, I, L, P, I, I, I, P],
-        "mgpt_expert_combine": [P, P, I, I, I, F, P],
+        "mgpt_expert_combine": [P, P, P, P, I, I, I, F, P],
     }
     for name, argtypes in table.items():
         fn = getattr(lib, name, None)

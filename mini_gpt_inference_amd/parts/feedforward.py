@@ -190,8 +190,11 @@ class TableExperts(FeedForward):
         plain_residual(ctx, h, x)
         n, ws = ctx.n_rows, ctx.workspace
         hn = as_tensor(ctx, h)
-        # tiles of 64 slots for the MFMA kernel, of 16 for the general one
         fast = not ctx.exact and ctx.dtype == torch.bfloat16
+        if fast and n * self.top >= self.TILED_FROM_PAIRS and self.width % 16 == 0 and self.hidden % 16 == 0 \
+                and self._forward_tiled(ctx, hn, x, n):
+            return
+        # tiles of 64 slots for the MFMA kernel of few rows, of 16 for the general one
         tile = 64 if fast else 16
         slots = kernels.expert_slots(n, self.top, self.n_experts, tile)
         slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
@@ -208,4 +211,38 @@ class TableExperts(FeedForward):
                                tile, fast)
         if self.shared_hidden:
             _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
-        kernels.expert_combine(pair_out, x, n, self.top, 1.0 / self.top)
+        kernels.expert_combine(pair_out, x, n, self.top, 1.0 / self.top, q_req=ctx.q_req)
+
+    # From this many (token, choice) pairs on, the experts' products go through the tiled MFMA kernel
+    # of the dense layers: the pairs' rows are copied into the experts' order first, every expert's
+    # run padded to whole tiles of 256 slots, so that a tile of that kernel multiplies one expert's
+    # matrix.  Below it a step is a decode step or a short portion, and padding every expert to 256
+    # rows would be most of the work.
+    TILED_FROM_PAIRS = 512
+
+    def _forward_tiled(self, ctx: StepContext, hn: torch.Tensor, x: torch.Tensor, n: int) -> bool:
+        ws, tile = ctx.workspace, 256
+        slots = kernels.expert_slots(n, self.top, self.n_experts, tile)
+        slot_token = ws.get("expert_slot_token", slots, 1, torch.int32).view(-1)
+        slot_pair = ws.get("expert_slot_pair", slots, 1, torch.int32).view(-1)
+        pair_slot = ws.get("expert_pair_slot", n * self.top, 1, torch.int32).view(-1)
+        tile_expert = ws.get("expert_tile", slots // tile, 1, torch.int32).view(-1)
+        sorted_rows = ws.get("expert_rows", slots, self.width, ctx.dtype)
+        if hn.stride(0) % 8 or hn.data_ptr() % 16 or sorted_rows.data_ptr() % 16:
+            return False
+        kernels.expert_route(ctx.token_ids, ctx.q_req, self.table, n, self.n_experts, slot_token, slot_pair,
+                             tile_expert, tile, pair_slot=pair_slot)
+        if not kernels.gather_rows(hn, slot_token, sorted_rows, slots):
+            return False
+        z = ws.get("expert_z", slots, 2 * self.hidden, ctx.dtype)
+        if not kernels.grouped_linear_tiled(sorted_rows, self.in_weights, tile_expert, slot_token, z, slots):
+            return False
+        act = ws.get("expert_act", slots, self.hidden, ctx.dtype)
+        kernels.gated_unit(z, act, slots, self.hidden, fast=True)
+        slot_out = ws.get("expert_slot_out", slots, self.width, torch.float32)
+        if not kernels.grouped_linear_tiled(act, self.down_weights, tile_expert, slot_token, slot_out, slots):
+            return False
+        if self.shared_hidden:
+            _gated(ctx, hn, self.shared_in_weight, self.shared_down, x, n, self.shared_hidden)
+        kernels.expert_combine(slot_out, x, n, self.top, 1.0 / self.top, pair_slot=pair_slot, q_req=ctx.q_req)
+        return True

@@ -123,7 +123,7 @@ def test_gated_unit(dtype):
 @pytest.mark.parametrize("dtype,tile,fast", [("float32", 16, False), ("bfloat16", 16, False), ("bfloat16", 64, True),
                                              ("float32", 64, False)])
 @pytest.mark.parametrize("n,experts,top,width,hidden", [(1, 2, 1, 24, 8), (40, 5, 2, 64, 24), (300, 16, 1, 48, 40),
-                                                        (7, 3, 3, 32, 16), (130, 4, 2, 100, 36)])
+                                                        (7, 3, 3, 32, 16), (130, 4, 2, 100, 36), (130, 4, 2, 64, 256), (70, 3, 1, 512, 40)])
 def test_experts_by_table(dtype, tile, fast, n, experts, top, width, hidden):
     """Route, both grouped products, the gated unit and the sum over a token's experts, against the
     plain loop; some tokens are padding (their request is -1) and an expert may get no token."""
@@ -162,6 +162,46 @@ def test_experts_by_table(dtype, tile, fast, n, experts, top, width, hidden):
     helpers.assert_close(y[live], want[live], dtype, "experts")
 
 
+@pytest.mark.parametrize("n,experts,top,width,hidden", [(700, 6, 2, 64, 96), (130, 4, 2, 64, 256), (1500, 8, 2, 128, 64),
+                                                        (40, 3, 1, 32, 16)])
+def test_experts_through_the_tiled_kernel(n, experts, top, width, hidden):
+    """The same with every expert's run padded to tiles of 256 slots: rows copied into the experts'
+    order, the dense layers' tiled MFMA kernel with a matrix per tile, and the sum through the
+    pairs' slots."""
+    g = torch.Generator().manual_seed(n)
+    vocab, tile = 31, 256
+    table = torch.rand(vocab, experts, generator=g).argsort(dim=1)[:, :top].to(torch.int32)
+    ids = torch.randint(0, vocab, (n,), generator=g, dtype=torch.int32)
+    q_req = torch.zeros(n, dtype=torch.int32)
+    q_req[-3:] = -1
+    h = _rnd(g, n, width, dtype="bfloat16")
+    w_in = _rnd(g, experts, 2 * hidden, width, dtype="bfloat16", scale=width ** -0.5)
+    w_down = _rnd(g, experts, width, hidden, dtype="bfloat16", scale=hidden ** -0.5)
+    slots = kernels.expert_slots(n, top, experts, tile)
+    st, sp = (torch.full((slots,), -7, dtype=torch.int32, device=DEV) for _ in range(2))
+    ps = torch.full((n * top,), -7, dtype=torch.int32, device=DEV)
+    te = torch.full((slots // tile,), -7, dtype=torch.int32, device=DEV)
+    kernels.expert_route(ids.to(DEV), q_req.to(DEV), table.to(DEV), n, experts, st, sp, te, tile, pair_slot=ps)
+    rows = torch.full((slots, width), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert kernels.gather_rows(h.to(DEV), st, rows, slots)
+    z = torch.full((slots, 2 * hidden), float("nan"), dtype=torch.bfloat16, device=DEV)
+    assert kernels.grouped_linear_tiled(rows, w_in.to(DEV), te, st, z, slots)
+    act = torch.zeros(slots, hidden, dtype=torch.bfloat16, device=DEV)
+    kernels.gated_unit(z, act, slots, hidden, fast=True)
+    out = torch.full((slots, width), float("nan"), device=DEV)
+    assert kernels.grouped_linear_tiled(act, w_down.to(DEV), te, st, out, slots)
+    y = torch.ones(n, width, device=DEV)
+    kernels.expert_combine(out, y, n, top, 1.0 / top, pair_slot=ps, q_req=q_req.to(DEV))
+    live = list(range(n - 3))
+    st_h, sp_h, ps_h = st.cpu(), sp.cpu(), ps.cpu()
+    assert all(int(sp_h[int(ps_h[p])]) == p and int(st_h[int(ps_h[p])]) == p // top for i in live for p in
+               range(i * top, (i + 1) * top))
+    exp = [(w_in[e, :hidden].float(), w_in[e, hidden:].float(), w_down[e].float()) for e in range(experts)]
+    want = 1.0 + V.table_moe(h.float(), ids.tolist(), table.long(), exp, None)
+    helpers.assert_close(y[live], want[live], "bfloat16", "experts, tiled")
+    assert (y[n - 3:] == 1.0).all(), "a padded token's row was touched"
+
+
 # ---------------------------------------------------------------- attention with sinks, kernel by kernel
 def _sink_want(c, sinks, scale, window):
     outs = []
@@ -187,6 +227,9 @@ SINK_CASES = [
     dict(seq_lens=[77, 150, 33], q_lens=[1, 1, 1], h=2, hk=1, d=40, page=16, window=33,
          spikes=[(0, 0, 44, 0), (1, 0, 117, 1), (2, 0, 0, 0)]),
     dict(seq_lens=[260], q_lens=[130], h=4, hk=1, d=128, page=32, window=129, spikes=[(0, 129, 131, 0), (0, 129, 130, 3)]),
+    # few tiles of a small head size: the tile kernel's two wave groups each see keys of their own
+    dict(seq_lens=[400], q_lens=[300], h=2, hk=1, d=32, page=16, window=0, spikes=[(0, 299, 5, 0), (0, 200, 240, 1)]),
+    dict(seq_lens=[700, 300], q_lens=[290, 300], h=3, hk=1, d=64, page=16, window=300, spikes=[(0, 289, 400, 0), (1, 150, 140, 1)]),
 ]
 
 
@@ -330,6 +373,27 @@ def test_long_decoding_past_every_window(tmp_path_factory, dtype):
         helpers.assert_close(got["a"], want, dtype, "long decoding")
     else:
         _assert_within_rounding(folder, "P", "long", ids, got["a"], want, "long decoding")
+
+
+def test_a_long_portion_takes_the_tiled_experts(tmp_path_factory, monkeypatch):
+    """A portion of 300 tokens with two experts each is beyond the bound from which the experts'
+    products go through the tiled kernel; the same prompt in short portions stays below it."""
+    folder = _folder(tmp_path_factory, "P")
+    ids = helpers.random_ids(np.random.default_rng(21), cases.RAW["P"]["vocab"], 300)
+    cfg, w = V.read_model_folder(folder)
+    want = V.forward(cfg, w, ids)[0].numpy()
+    calls = []
+    tiled = kernels.grouped_linear_tiled
+    monkeypatch.setattr(kernels, "grouped_linear_tiled", lambda *a, **k: calls.append(1) or tiled(*a, **k))
+    for cut in (300, 60):
+        plan = helpers.TracePlan()
+        for at in range(0, 300, cut):
+            plan.add_step([("a", ids[at:at + cut], 300)], end=["a"] if at + cut >= 300 else [])
+        replayer = TraceReplayer(folder, "bfloat16", 320, page_size=16, max_live=4, poison=True)
+        before = len(calls)
+        got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {"a": 300}, cases.RAW["P"]["vocab"])
+        assert (len(calls) > before) == (cut == 300)
+        _assert_within_rounding(folder, "P", "tiled", ids, got["a"], want, f"portions of {cut}")
 
 
 def test_the_sink_and_the_far_latents_matter(tmp_path_factory, tmp_path):

@@ -46,7 +46,7 @@ RAW: Dict[str, dict] = {
     "P": {"architecture": "Viperax", "vocab": 131, "width": 64, "streams": 2, "norm": {"eps": 1e-5},
           "embedding": {"scale": 8.0}, "logit_scale": 0.5, "logit_softcap": 10.0,
           "layers": [_layer(_mixer(2, 16, 32, 32, 0.3, window=9), {"kind": "dense", "ff": 48}),
-                     _layer(_mixer(2, 16, 32, 32, 0.3, window=20), _moe(24, 5, 2, shared=40)),
+                     _layer(_mixer(2, 16, 32, 32, 0.3, window=20), _moe(32, 5, 2, shared=40)),
                      _layer(_mixer(4, 8, 16, 32, 0.4, window=33, kv_from=1), None),
                      _layer(_mixer(2, 16, 32, 32, 0.3, kv_from=0), _moe(16, 3, 1))]},
     # one stream with hyper-connection tensors, one head, top 1 of 2, a window of one token, a latent
