@@ -301,7 +301,8 @@ extern "C" int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_ro
     return MGPT_ERR_BAD_SHAPE;
   if (n_tiles > 65535) return MGPT_ERR_TOO_LARGE;
   // wide outputs: a wave takes 64 columns; narrow ones 16, so that a tile still gives several workgroups
-  const bool wide = n_out >= 512;
+  // ... and so do few tiles (a decode step): more workgroups then walk the inner size side by side
+  const bool wide = n_out >= 512 && n_tiles >= 64;
   dim3 grid((n_out + (wide ? 255 : 63)) / (wide ? 256 : 64), n_tiles), block(256);
 #define GM_LAUNCH(OT, NJ)                                                                                     \
   hipLaunchKernelGGL((grouped_linear_mfma_kernel<OT, NJ>), grid, block, 0, stream, (const bf16_t*)a, lda,     \

@@ -117,6 +117,9 @@ int mgpt_streams_read(const float* x, const float* coef, float* u, float* zero, 
     streams, hipStream_t stream);
 int mgpt_streams_write(float* x, const float* mix, const float* out, const float* y, int n_rows, int width, int
     streams, hipStream_t stream);
+int mgpt_streams_step(float* x, const float* mix, const float* out, float* y, int fold, int clear, const float*
+    coef, float* u, const float* gain, const float* beta, float eps, void* h, int h_dtype, int n_rows, int width,
+    int streams, hipStream_t stream);
 int mgpt_scale_softcap(float* logits, long ld, int n_rows, int vocab, float scale, float cap, int fast,
     hipStream_t stream);
 // latent.hip
@@ -177,6 +180,7 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_embed_scaled) \
   X(mgpt_streams_read) \
   X(mgpt_streams_write) \
+  X(mgpt_streams_step) \
   X(mgpt_scale_softcap) \
   X(mgpt_rms_norm_store) \
   X(mgpt_heads_linear) \

@@ -108,6 +108,143 @@ extern "C" int mgpt_streams_write(float* x, const float* mix, const float* out, 
   return mgpt_last_error();
 }
 
+// A sublayer's write, the next sublayer's read and its LayerNorm in one pass over a token's streams:
+//   x[t] <- sum_s mix[s][t] x[s] + out[t] y   (left out when y is null: the streams are as they are)
+//   y <- 0                                      (the next sublayer adds its output into it)
+//   u = sum_t coef[t] x[t];  h = (u - mean) / sqrt(var + eps) * gain (+ beta)
+// One workgroup a token; a thread keeps its share of u in registers (widths up to 256 * SS_KEEP,
+// wider rows are read back from `u`).  Mean first, then the centred squares, as the LayerNorm kernel.
+#define SS_KEEP 16
+
+__device__ __forceinline__ float ss_block_sum(float v, float* red) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();   // the last use of red is over
+  if (lane == 0) red[wave] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+template <typename OT>
+__global__ __launch_bounds__(256) void streams_step_kernel(
+    float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ out, float* __restrict__ y,
+    int fold, int clear, const float* __restrict__ coef, float* __restrict__ u, const float* __restrict__ gain,
+    const float* __restrict__ beta, float eps, OT* __restrict__ h, int width, int streams) {
+  __shared__ float red[4];
+  __shared__ float m_s[MGPT_MAX_STREAMS * MGPT_MAX_STREAMS], o_s[MGPT_MAX_STREAMS], c_s[MGPT_MAX_STREAMS];
+  const int tid = threadIdx.x;
+  const long n = blockIdx.x;
+  if (tid < streams * streams) m_s[tid] = fold ? mix[tid] : 0.f;
+  if (tid < streams) {
+    o_s[tid] = fold ? out[tid] : 0.f;
+    c_s[tid] = coef[tid];
+  }
+  __syncthreads();
+  float* xr = x + n * (long)streams * width;
+  // column c of the token, from its old streams and y: the streams rewritten (if a write is pending),
+  // y cleared, u returned
+  auto column = [&](int c, const float* old, float yv) -> float {
+    float uv = 0.f;
+    if (fold) {
+      for (int t = 0; t < streams; ++t) {
+        float acc = 0.f;
+#pragma unroll
+        for (int s = 0; s < MGPT_MAX_STREAMS; ++s)
+          if (s < streams) acc = fmaf(m_s[s * streams + t], old[s], acc);
+        acc = fmaf(o_s[t], yv, acc);
+        xr[(long)t * width + c] = acc;
+        uv = fmaf(c_s[t], acc, uv);
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < MGPT_MAX_STREAMS; ++s)
+        if (s < streams) uv = fmaf(c_s[s], old[s], uv);
+    }
+    if (clear) y[n * width + c] = 0.f;
+    u[n * width + c] = uv;
+    return uv;
+  };
+  auto load = [&](int c, float* old, float& yv) {
+#pragma unroll
+    for (int s = 0; s < MGPT_MAX_STREAMS; ++s) old[s] = s < streams ? xr[(long)s * width + c] : 0.f;
+    yv = fold ? y[n * width + c] : 0.f;
+  };
+  float keep[SS_KEEP];
+  float sum = 0.f;
+  // four columns at a time: all their loads are asked for before the first of them is waited for
+#pragma unroll
+  for (int i0 = 0; i0 < SS_KEEP; i0 += 4) {
+    float old[4][MGPT_MAX_STREAMS], yv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = tid + (i0 + j) * 256;
+      load(c < width ? c : 0, old[j], yv[j]);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int c = tid + (i0 + j) * 256;
+      keep[i0 + j] = c < width ? column(c, old[j], yv[j]) : 0.f;
+      sum += keep[i0 + j];
+    }
+  }
+  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+    float old[MGPT_MAX_STREAMS], yv;
+    load(c, old, yv);
+    sum += column(c, old, yv);
+  }
+  const float mean = ss_block_sum(sum, red) / (float)width;
+  float e = 0.f, v2 = 0.f;
+#pragma unroll
+  for (int i = 0; i < SS_KEEP; ++i) {
+    const float d = tid + i * 256 < width ? keep[i] - mean : 0.f;
+    keep[i] = d;
+    e += d;
+    v2 = fmaf(d, d, v2);
+  }
+  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+    const float d = u[n * width + c] - mean;
+    e += d;
+    v2 = fmaf(d, d, v2);
+  }
+  const float corr = ss_block_sum(e, red) / (float)width;
+  const float var = fmaxf(ss_block_sum(v2, red) / (float)width - corr * corr, 0.f);
+  const float rstd = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int i = 0; i < SS_KEEP; ++i) {
+    const int c = tid + i * 256;
+    if (c < width) {
+      float v = (keep[i] - corr) * rstd * gain[c];
+      if (beta) v += beta[c];
+      h[n * width + c] = from_float<OT>(v);
+    }
+  }
+  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+    float v = ((u[n * width + c] - mean) - corr) * rstd * gain[c];
+    if (beta) v += beta[c];
+    h[n * width + c] = from_float<OT>(v);
+  }
+}
+
+// y [n_rows, width]: with fold, the output of the sublayer whose write is still to be made (without, the
+// streams are read as they are); with clear, it is zero afterwards.  u: float32 [n_rows, width]; h:
+// [n_rows, width] in h_dtype.  x, y, u and h are four different buffers.
+extern "C" int mgpt_streams_step(float* x, const float* mix, const float* out, float* y, int fold, int clear,
+                                 const float* coef, float* u, const float* gain, const float* beta, float eps, void* h,
+                                 int h_dtype, int n_rows, int width, int streams, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!x || !coef || !u || !gain || !h || (fold && (!mix || !out)) || ((fold || clear) && !y)) return MGPT_ERR_NULL;
+  if (n_rows < 0 || width <= 0 || streams <= 0 || streams > MGPT_MAX_STREAMS) return MGPT_ERR_BAD_SHAPE;
+  if (h_dtype == MGPT_F32)
+    hipLaunchKernelGGL(streams_step_kernel<float>, dim3(n_rows), dim3(256), 0, stream, x, mix, out, y, fold, clear, coef, u,
+                       gain, beta, eps, (float*)h, width, streams);
+  else if (h_dtype == MGPT_BF16)
+    hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, stream, x, mix, out, y, fold, clear, coef, u,
+                       gain, beta, eps, (bf16_t*)h, width, streams);
+  else
+    return MGPT_ERR_BAD_DTYPE;
+  return mgpt_last_error();
+}
+
 template <bool FAST>
 __global__ void scale_softcap_kernel(float* __restrict__ logits, long ld, int n_rows, int vocab, float scale,
                                      float cap) {

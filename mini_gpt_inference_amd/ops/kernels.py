@@ -989,6 +989,36 @@ def streams_write(x: torch.Tensor, mix: torch.Tensor, out: torch.Tensor, y: torc
     _check(rc, "streams_write")
 
 
+def streams_step(x: torch.Tensor, write, coef: torch.Tensor, u: torch.Tensor, gain: torch.Tensor,
+                 beta: Optional[torch.Tensor], eps: float, h: torch.Tensor, n_rows: int, streams: int,
+                 zero: Optional[torch.Tensor] = None) -> None:
+    """One pass over every token's streams: the write that is still to be made (write = (mix, out, y)
+    as for streams_write, or None), `zero` cleared (it may be y), then u = sum_t coef[t] x[t] and
+    h = LayerNorm(u) with gain (and beta), in h's dtype."""
+    mix, out, y = write if write is not None else (None, None, None)
+    _need_cuda(x, mix, out, y, coef, u, gain, beta, h, zero)
+    width = u.shape[1]
+    _need_streams(x, n_rows, width, streams)
+    _need_rows_f32("u", u, n_rows, width)
+    for name, t in (("y", y), ("zero", zero)):
+        if t is not None:
+            _need_rows_f32(name, t, n_rows, width)
+    _need(h.dim() == 2 and h.is_contiguous() and h.shape[1] == width and h.shape[0] >= n_rows, "h must be dense [>=n_rows, width]")
+    _need(coef.dtype == torch.float32 and coef.is_contiguous() and coef.numel() == streams, "coef must be float32 [streams]")
+    if write is not None:
+        _need(mix.dtype == torch.float32 and mix.is_contiguous() and tuple(mix.shape) == (streams, streams)
+              and out.dtype == torch.float32 and out.is_contiguous() and out.numel() == streams,
+              "mix must be float32 [streams, streams] and out float32 [streams]")
+    _need(gain.dtype == torch.float32 and gain.numel() == width and (beta is None or (beta.dtype == torch.float32
+          and beta.numel() == width)), "gain and beta must be float32 [width]")
+    _need(y is None or zero is None or y.data_ptr() == zero.data_ptr(), "the buffer to clear is y itself")
+    buf = y if y is not None else zero
+    rc = library.kernels().mgpt_streams_step(_ptr(x), _ptr(mix), _ptr(out), _ptr(buf), int(write is not None),
+                                             int(zero is not None), _ptr(coef), _ptr(u), _ptr(gain), _ptr(beta),
+                                             float(eps), _ptr(h), _dtype_code(h), n_rows, width, streams, _stream())
+    _check(rc, "streams_step")
+
+
 def scale_softcap(logits: torch.Tensor, n_rows: int, scale: float, cap: float, fast: bool) -> None:
     """logits = cap * tanh(logits * scale / cap) in place (cap <= 0: the scale alone)."""
     _need_cuda(logits)

@@ -151,6 +151,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_embed_scaled": [P, P, P, I, I, I, F, I, P],
         "mgpt_streams_read": [P, P, P, P, I, I, I, P],
         "mgpt_streams_write": [P, P, P, P, I, I, I, P],
+        "mgpt_streams_step": [P, P, P, P, I, I, P, P, P, P, F, P, I, I, I, I, P],
         "mgpt_scale_softcap": [P, L, I, I, F, F, I, P],
         # latent attention
         "mgpt_rms_norm_store": [P, I, L, P, F, P, P, I, I, P],

@@ -205,6 +205,9 @@ class StepContext:
     # an ops.linear.CopyBudget: device memory that copies of matrices made at first use may still take;
     # None: no bound
     copy_budget: Optional[Any] = None
+    # a write into the residual streams that its arrangement has left to the next reader of the streams:
+    # (mix, out, y) as for ops.kernels.streams_write; None: the streams are up to date
+    pending_streams: Optional[Any] = None
     # set by a caller that will choose greedily among the logits: an ops.linear.TileBest, which the
     # head fills beside the logits if its kernel can
     tile_best: Optional[Any] = None

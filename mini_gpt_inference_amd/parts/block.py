@@ -55,6 +55,14 @@ class PreNorm(Arrangement):
         feed_forward.forward_add(ctx, LazyNorm(norm2, x, n), x)
 
 
+def flush_streams(ctx: StepContext, x: torch.Tensor, streams: int) -> None:
+    """Makes the write into the residual streams that a sublayer has left pending, if any."""
+    if ctx.pending_streams is not None:
+        mix, out, y = ctx.pending_streams
+        ctx.pending_streams = None
+        kernels.streams_write(x, mix, out, y, ctx.n_rows, streams)
+
+
 @register_arrangement("hyper_connections")
 class HyperConnections(Arrangement):
     """A pre-norm layer over several residual streams.  A token's residual is S rows x_1 .. x_S.
@@ -65,7 +73,9 @@ class HyperConnections(Arrangement):
 
     every new stream from the old ones, all in float32.  With S = 1, a = b = 1 and M = 1 this is
     the plain pre-norm layer.  The sublayers are the framework's ordinary parts: they add their
-    output into a cleared buffer that stands for y."""
+    output into a cleared buffer that stands for y.  A sublayer's write is left pending
+    (ctx.pending_streams) and made by the kernel that reads the streams next: the next sublayer's
+    read and LayerNorm, or the model before the final norm."""
 
     graph_safe = True
     plan_safe = True
@@ -85,13 +95,27 @@ class HyperConnections(Arrangement):
             req["mix" + q] = WeightRequest((s, s), VECTOR)
         return req
 
+    # the arrangement reads ctx.pending_streams: a write that the sublayer before (of this layer or of
+    # the one before) has left to be made together with this sublayer's read
+    takes_pending_streams = True
+
     def _sublayer(self, ctx: StepContext, x: torch.Tensor, q: str, norm: Part, call) -> None:
         n, ws = ctx.n_rows, ctx.workspace
         u = ws.get("streams_read", n, self.width, torch.float32)
         y = ws.get("streams_update", n, self.width, torch.float32)
-        kernels.streams_read(x, getattr(self, "in" + q), u, n, self.streams, zero=y)
-        call(LazyNorm(norm, u, n), y)
-        kernels.streams_write(x, getattr(self, "mix" + q), getattr(self, "out" + q), y, n, self.streams)
+        if getattr(norm, "fusable_layer_norm", False):
+            # one kernel: the write left over from the sublayer before, y cleared, this sublayer's
+            # read and its LayerNorm
+            h = ws.get("normed", n, self.width, ctx.dtype)
+            kernels.streams_step(x, ctx.pending_streams, getattr(self, "in" + q), u, norm.weight, norm.bias, norm.eps,
+                                 h, n, self.streams, zero=y)
+            ctx.pending_streams = None
+        else:
+            flush_streams(ctx, x, self.streams)
+            kernels.streams_read(x, getattr(self, "in" + q), u, n, self.streams, zero=y)
+            h = LazyNorm(norm, u, n)
+        call(h, y)
+        ctx.pending_streams = (getattr(self, "mix" + q), getattr(self, "out" + q), y)
 
     def run(self, ctx, x, parts, bindings, position) -> None:
         mixer = parts["mixer"]

@@ -353,12 +353,16 @@ class DecoderModel:
         streams = self.spec.streams
         x = ws.get("residual", n, streams * self.spec.width, torch.float32)
         ctx.pending = None
+        ctx.pending_streams = None
         self.embedding.forward(ctx, self.position, x)
         for run, bindings in zip(self.spec.order, self.cache_layout.run_bindings):
             layer = self.layers[run.layer]
+            if not getattr(layer.arrangement, "takes_pending_streams", False):
+                _block.flush_streams(ctx, x, streams)
             if not layer.arrangement.takes_pending_residual:
                 residual.settle(ctx, x, n)
             layer.arrangement.run(ctx, x, layer.parts, bindings, self.position)
+        _block.flush_streams(ctx, x, streams)
         if streams > 1:
             # the streams' sum is what the final norm reads
             total = ws.get("residual_sum", n, self.spec.width, torch.float32)

@@ -51,6 +51,31 @@ def test_streams_read_and_write(streams, width, n):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("streams,width,n", [(1, 40, 3), (2, 64, 70), (3, 192, 9), (4, 4100, 2), (2, 5000, 3)])
+def test_streams_write_read_and_norm_in_one_pass(dtype, streams, width, n):
+    g = torch.Generator().manual_seed(streams + width)
+    x = _rnd(g, n + 1, streams * width, scale=3.0)
+    coef, out, mix = _rnd(g, streams), _rnd(g, streams), _rnd(g, streams, streams)
+    gain, beta = _rnd(g, width) + 1.0, _rnd(g, width)
+    y = _rnd(g, n + 1, width)
+    as_streams = x[:n].view(n, streams, width).transpose(0, 1)
+    for pending in (False, True):
+        xd, yd = x.to(DEV), y.to(DEV)
+        u = torch.zeros(n + 1, width, device=DEV)
+        h = torch.full((n + 1, width), 5.0, dtype=TDT[dtype], device=DEV)
+        kernels.streams_step(xd, (mix.to(DEV), out.to(DEV), yd) if pending else None, coef.to(DEV), u, gain.to(DEV),
+                             beta.to(DEV) if pending else None, 1e-5, h, n, streams, zero=yd)
+        new = V.hyper_write(as_streams, mix, out, y[:n]) if pending else as_streams
+        helpers.assert_close(xd[:n], new.transpose(0, 1).reshape(n, streams * width), "float32", "streams")
+        want_u = V.hyper_read(new, coef)
+        helpers.assert_close(u[:n], want_u, "float32", "u")
+        want_h = V.layer_norm(want_u, gain, 1e-5) + (beta if pending else 0.0)
+        helpers.assert_close(h[:n], want_h, dtype, "normed")
+        assert (yd[:n] == 0).all() and torch.equal(yd[n:].cpu(), y[n:]) and (h[n:] == 5.0).all()
+        assert torch.equal(xd[n:].cpu(), x[n:])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_embed_scaled_fills_every_stream(dtype):
     g = torch.Generator().manual_seed(1)
     table = _rnd(g, 50, 36, dtype=dtype)
