@@ -331,16 +331,41 @@ __global__ void expert_combine_kernel(const float* __restrict__ pair_out, const 
   y[i] += acc * weight;
 }
 
+// the same, four columns a thread (widths in steps of 4, 16-byte aligned buffers)
+__global__ void expert_combine4_kernel(const float4* __restrict__ pair_out, const int* __restrict__ pair_slot,
+                                       const int* __restrict__ q_req, float4* __restrict__ y, long total, int width4,
+                                       int top, float weight) {
+  const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const long n = i / width4;
+  const int c = (int)(i - n * width4);
+  if (q_req && q_req[n] < 0) return;
+  float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int k = 0; k < top; ++k) {
+    const long row = pair_slot ? pair_slot[n * top + k] : n * top + k;
+    const float4 v = pair_out[row * (long)width4 + c];
+    acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+  }
+  float4 o = y[i];
+  o.x += acc.x * weight; o.y += acc.y * weight; o.z += acc.z * weight; o.w += acc.w * weight;
+  y[i] = o;
+}
+
 // y[n] += weight * sum_k pair_out[pair_slot[n * top + k]] (pair_slot null: row n * top + k itself)
 extern "C" int mgpt_expert_combine(const float* pair_out, const int* pair_slot, const int* q_req, float* y, int n_rows,
                                    int width, int top, float weight, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!pair_out || !y) return MGPT_ERR_NULL;
   if (n_rows < 0 || width <= 0 || top <= 0) return MGPT_ERR_BAD_SHAPE;
-  const long total = (long)n_rows * width;
+  const bool vec = (width & 3) == 0 && ((((size_t)pair_out) | ((size_t)y)) & 15) == 0;
+  const long total = (long)n_rows * (vec ? width / 4 : width);
   const long blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(expert_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, pair_out, pair_slot, q_req, y,
-                     total, width, top, weight);
+  if (vec)
+    hipLaunchKernelGGL(expert_combine4_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (const float4*)pair_out,
+                       pair_slot, q_req, (float4*)y, total, width / 4, top, weight);
+  else
+    hipLaunchKernelGGL(expert_combine_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, pair_out, pair_slot, q_req, y,
+                       total, width, top, weight);
   return mgpt_last_error();
 }

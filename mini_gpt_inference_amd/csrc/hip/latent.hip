@@ -114,23 +114,30 @@ extern "C" int mgpt_heads_linear(const void* a, long lda, const void* w, void* o
   return mgpt_last_error();
 }
 
-// The same products in bfloat16 on the MFMA units.  A workgroup (four waves) owns 64 rows x 64
-// columns of one head; a wave owns 16 of the columns for all 64 rows: per 32 k it loads its
-// slice of the head's matrix once (the first MFMA operand, 16 bytes a lane straight from memory)
-// and four slices of the rows, and a lane ends up with four neighbouring columns of one row in
-// each of its four results.  Inner sizes in steps of 8, outputs in steps of 4.
+// The same products in bfloat16 on the MFMA units.  A wave owns 64 rows x up to 128 columns of one
+// head (a workgroup, four waves, 256 rows): per 32 k it loads the slices of the head's matrix for
+// its columns (the first MFMA operand, 16 bytes a lane straight from memory; a head's matrix is a
+// few KB and stays in the cache) and four slices of the rows, and a lane ends up with four
+// neighbouring columns of one row in each result.  Inner sizes in steps of 8, outputs in steps of 4.
 typedef __attribute__((__vector_size__(8 * sizeof(short)))) short hl_bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hl_f32x4_t;
 
+template <int NJ>
 __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
     const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, bf16_t* __restrict__ out, long ldo,
     const bf16_t* __restrict__ gate, long ldg, int n_rows, int n_out, int k_dim) {
+  // a wave owns 64 rows x NJ * 16 columns of one head: the rows are read once for all those columns
   const int head = blockIdx.z, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int row0 = blockIdx.y * 64, col0 = blockIdx.x * 64 + wave * 16;
-  if (col0 >= n_out) return;   // the whole wave; the kernel has no barrier
+  const int row0 = (blockIdx.y * 4 + wave) * 64, col0 = blockIdx.x * (NJ * 16);
+  if (row0 >= n_rows) return;   // the whole wave; the kernel has no barrier
   const int li = lane & 15, lg = lane >> 4;
-  const bool w_ok = col0 + li < n_out;
-  const bf16_t* wrow = W + ((long)head * n_out + (w_ok ? col0 + li : 0)) * (long)k_dim;
+  const bf16_t* wrow[NJ];
+  bool w_ok[NJ];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    w_ok[j] = col0 + j * 16 + li < n_out;
+    wrow[j] = W + ((long)head * n_out + (w_ok[j] ? col0 + j * 16 + li : 0)) * (long)k_dim;
+  }
   const bf16_t* arow[4];
   bool a_ok[4];
 #pragma unroll
@@ -140,38 +147,48 @@ __global__ __launch_bounds__(256) void heads_linear_mfma_kernel(
     arow[t] = A + (long)(a_ok[t] ? r : 0) * lda + (long)head * k_dim;
   }
   const hl_bf16x8_t zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  hl_f32x4_t acc[4];
+  hl_f32x4_t acc[NJ][4];
 #pragma unroll
-  for (int t = 0; t < 4; ++t) acc[t] = hl_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < NJ; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) acc[j][t] = hl_f32x4_t{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < k_dim; k0 += 32) {
     const int k = k0 + lg * 8;
     const bool k_ok = k < k_dim;
-    const hl_bf16x8_t wf = (w_ok && k_ok) ? *reinterpret_cast<const hl_bf16x8_t*>(wrow + k) : zero;
-    hl_bf16x8_t af[4];
+    hl_bf16x8_t wf[NJ], af[4];
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+      wf[j] = (w_ok[j] && k_ok) ? *reinterpret_cast<const hl_bf16x8_t*>(wrow[j] + k) : zero;
 #pragma unroll
     for (int t = 0; t < 4; ++t)
       af[t] = (a_ok[t] && k_ok) ? *reinterpret_cast<const hl_bf16x8_t*>(arow[t] + k) : zero;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, af[t], acc[t], 0, 0, 0);
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int t = 0; t < 4; ++t)
+        acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[j], af[t], acc[j][t], 0, 0, 0);
   }
-  const int c = col0 + lg * 4;   // this lane's four columns, of row 16 t + li
-  if (c >= n_out) return;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int r = row0 + 16 * t + li;
-    if (r >= n_rows) continue;
-    float v[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
-    if (gate) {
-      const uint2 g = *reinterpret_cast<const uint2*>(gate + (long)r * ldg + (long)head * n_out + c);
-      const float gv[4] = {bf16_to_float((bf16_t)(g.x & 0xffff)), bf16_to_float((bf16_t)(g.x >> 16)),
-                           bf16_to_float((bf16_t)(g.y & 0xffff)), bf16_to_float((bf16_t)(g.y >> 16))};
+  for (int j = 0; j < NJ; ++j) {
+    const int c = col0 + j * 16 + lg * 4;   // this lane's four columns, of row 16 t + li
+    if (c >= n_out) continue;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] *= __builtin_amdgcn_rcpf(1.0f + __expf(-gv[i]));
+    for (int t = 0; t < 4; ++t) {
+      const int r = row0 + 16 * t + li;
+      if (r >= n_rows) continue;
+      float v[4] = {acc[j][t][0], acc[j][t][1], acc[j][t][2], acc[j][t][3]};
+      if (gate) {
+        const uint2 g = *reinterpret_cast<const uint2*>(gate + (long)r * ldg + (long)head * n_out + c);
+        const float gv[4] = {bf16_to_float((bf16_t)(g.x & 0xffff)), bf16_to_float((bf16_t)(g.x >> 16)),
+                             bf16_to_float((bf16_t)(g.y & 0xffff)), bf16_to_float((bf16_t)(g.y >> 16))};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] *= __builtin_amdgcn_rcpf(1.0f + __expf(-gv[i]));
+      }
+      uint2 pk;
+      pk.x = pack_bf16x2(v[0], v[1]);
+      pk.y = pack_bf16x2(v[2], v[3]);
+      *reinterpret_cast<uint2*>(out + (long)r * ldo + (long)head * n_out + c) = pk;
     }
-    uint2 pk;
-    pk.x = pack_bf16x2(v[0], v[1]);
-    pk.y = pack_bf16x2(v[2], v[3]);
-    *reinterpret_cast<uint2*>(out + (long)r * ldo + (long)head * n_out + c) = pk;
   }
 }
 
@@ -188,9 +205,21 @@ extern "C" int mgpt_heads_linear_mfma(const void* a, long lda, const void* w, vo
   if ((k_dim & 7) || (n_out & 3) || (lda & 7) || (ldo & 3) || (gate && (ldg & 3)) || (((size_t)a | (size_t)w) & 15) ||
       (((size_t)out | (size_t)gate) & 7))
     return MGPT_ERR_BAD_SHAPE;
-  if (n_head > 65535 || (n_rows + 63) / 64 > 65535) return MGPT_ERR_TOO_LARGE;
-  dim3 grid((n_out + 63) / 64, (n_rows + 63) / 64, n_head), block(256);
-  hipLaunchKernelGGL(heads_linear_mfma_kernel, grid, block, 0, stream, (const bf16_t*)a, lda, (const bf16_t*)w,
-                     (bf16_t*)out, ldo, (const bf16_t*)gate, ldg, n_rows, n_out, k_dim);
+  if (n_head > 65535 || (n_rows + 255) / 256 > 65535) return MGPT_ERR_TOO_LARGE;
+  // columns a wave, in sixteens: as many as still leave about a thousand waves (a wave's rows are read
+  // once for all of its columns), one sixteen where the rows are few
+  int nj = 8;
+  while (nj > 1 && (nj * 16 > n_out + 15 ||
+                    (long)((n_rows + 63) / 64) * ((n_out + nj * 16 - 1) / (nj * 16)) * n_head < 1024))
+    nj >>= 1;
+  dim3 grid((n_out + nj * 16 - 1) / (nj * 16), (n_rows + 255) / 256, n_head), block(256);
+#define HM_LAUNCH(NJ)                                                                                        \
+  hipLaunchKernelGGL(heads_linear_mfma_kernel<NJ>, grid, block, 0, stream, (const bf16_t*)a, lda,            \
+                     (const bf16_t*)w, (bf16_t*)out, ldo, (const bf16_t*)gate, ldg, n_rows, n_out, k_dim)
+  if (nj == 1) HM_LAUNCH(1);
+  else if (nj == 2) HM_LAUNCH(2);
+  else if (nj == 4) HM_LAUNCH(4);
+  else HM_LAUNCH(8);
+#undef HM_LAUNCH
   return mgpt_last_error();
 }

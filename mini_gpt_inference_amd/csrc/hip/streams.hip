@@ -112,25 +112,31 @@ extern "C" int mgpt_streams_write(float* x, const float* mix, const float* out, 
 //   x[t] <- sum_s mix[s][t] x[s] + out[t] y   (left out when y is null: the streams are as they are)
 //   y <- 0                                      (the next sublayer adds its output into it)
 //   u = sum_t coef[t] x[t];  h = (u - mean) / sqrt(var + eps) * gain (+ beta)
-// One workgroup a token; a thread keeps its share of u in registers (widths up to 256 * SS_KEEP,
+// One workgroup a token; a thread keeps its share of u in registers (up to SS_KEEP columns a thread,
 // wider rows are read back from `u`).  Mean first, then the centred squares, as the LayerNorm kernel.
 #define SS_KEEP 16
 
+template <int T>
 __device__ __forceinline__ float ss_block_sum(float v, float* red) {
   v = wave_sum(v);
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   __syncthreads();   // the last use of red is over
   if (lane == 0) red[wave] = v;
   __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < T / 64; ++w) total += red[w];
+  return total;
 }
 
-template <typename OT>
-__global__ __launch_bounds__(256) void streams_step_kernel(
+// T threads a token: 256 for a step of many tokens, 1024 for few (a decode step), where a token's
+// columns should be few a thread so that one round of loads covers them.
+template <typename OT, int T>
+__global__ __launch_bounds__(T) void streams_step_kernel(
     float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ out, float* __restrict__ y,
     int fold, int clear, const float* __restrict__ coef, float* __restrict__ u, const float* __restrict__ gain,
     const float* __restrict__ beta, float eps, OT* __restrict__ h, int width, int streams) {
-  __shared__ float red[4];
+  __shared__ float red[T / 64];
   __shared__ float m_s[MGPT_MAX_STREAMS * MGPT_MAX_STREAMS], o_s[MGPT_MAX_STREAMS], c_s[MGPT_MAX_STREAMS];
   const int tid = threadIdx.x;
   const long n = blockIdx.x;
@@ -177,48 +183,48 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
     float old[4][MGPT_MAX_STREAMS], yv[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int c = tid + (i0 + j) * 256;
+      const int c = tid + (i0 + j) * T;
       load(c < width ? c : 0, old[j], yv[j]);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int c = tid + (i0 + j) * 256;
+      const int c = tid + (i0 + j) * T;
       keep[i0 + j] = c < width ? column(c, old[j], yv[j]) : 0.f;
       sum += keep[i0 + j];
     }
   }
-  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+  for (int c = tid + SS_KEEP * T; c < width; c += T) {
     float old[MGPT_MAX_STREAMS], yv;
     load(c, old, yv);
     sum += column(c, old, yv);
   }
-  const float mean = ss_block_sum(sum, red) / (float)width;
+  const float mean = ss_block_sum<T>(sum, red) / (float)width;
   float e = 0.f, v2 = 0.f;
 #pragma unroll
   for (int i = 0; i < SS_KEEP; ++i) {
-    const float d = tid + i * 256 < width ? keep[i] - mean : 0.f;
+    const float d = tid + i * T < width ? keep[i] - mean : 0.f;
     keep[i] = d;
     e += d;
     v2 = fmaf(d, d, v2);
   }
-  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+  for (int c = tid + SS_KEEP * T; c < width; c += T) {
     const float d = u[n * width + c] - mean;
     e += d;
     v2 = fmaf(d, d, v2);
   }
-  const float corr = ss_block_sum(e, red) / (float)width;
-  const float var = fmaxf(ss_block_sum(v2, red) / (float)width - corr * corr, 0.f);
+  const float corr = ss_block_sum<T>(e, red) / (float)width;
+  const float var = fmaxf(ss_block_sum<T>(v2, red) / (float)width - corr * corr, 0.f);
   const float rstd = 1.0f / sqrtf(var + eps);
 #pragma unroll
   for (int i = 0; i < SS_KEEP; ++i) {
-    const int c = tid + i * 256;
+    const int c = tid + i * T;
     if (c < width) {
       float v = (keep[i] - corr) * rstd * gain[c];
       if (beta) v += beta[c];
       h[n * width + c] = from_float<OT>(v);
     }
   }
-  for (int c = tid + SS_KEEP * 256; c < width; c += 256) {
+  for (int c = tid + SS_KEEP * T; c < width; c += T) {
     float v = ((u[n * width + c] - mean) - corr) * rstd * gain[c];
     if (beta) v += beta[c];
     h[n * width + c] = from_float<OT>(v);
@@ -234,14 +240,14 @@ extern "C" int mgpt_streams_step(float* x, const float* mix, const float* out, f
   if (n_rows == 0) return MGPT_OK;
   if (!x || !coef || !u || !gain || !h || (fold && (!mix || !out)) || ((fold || clear) && !y)) return MGPT_ERR_NULL;
   if (n_rows < 0 || width <= 0 || streams <= 0 || streams > MGPT_MAX_STREAMS) return MGPT_ERR_BAD_SHAPE;
-  if (h_dtype == MGPT_F32)
-    hipLaunchKernelGGL(streams_step_kernel<float>, dim3(n_rows), dim3(256), 0, stream, x, mix, out, y, fold, clear, coef, u,
-                       gain, beta, eps, (float*)h, width, streams);
-  else if (h_dtype == MGPT_BF16)
-    hipLaunchKernelGGL(streams_step_kernel<bf16_t>, dim3(n_rows), dim3(256), 0, stream, x, mix, out, y, fold, clear, coef, u,
-                       gain, beta, eps, (bf16_t*)h, width, streams);
-  else
-    return MGPT_ERR_BAD_DTYPE;
+  const bool few = n_rows <= 128 && width > 1024;   // more than four columns a thread otherwise
+#define SS_LAUNCH(OT, T)                                                                                          \
+  hipLaunchKernelGGL((streams_step_kernel<OT, T>), dim3(n_rows), dim3(T), 0, stream, x, mix, out, y, fold, clear, \
+                     coef, u, gain, beta, eps, (OT*)h, width, streams)
+  if (h_dtype == MGPT_F32) { if (few) SS_LAUNCH(float, 1024); else SS_LAUNCH(float, 256); }
+  else if (h_dtype == MGPT_BF16) { if (few) SS_LAUNCH(bf16_t, 1024); else SS_LAUNCH(bf16_t, 256); }
+  else return MGPT_ERR_BAD_DTYPE;
+#undef SS_LAUNCH
   return mgpt_last_error();
 }
 

@@ -51,7 +51,8 @@ def test_streams_read_and_write(streams, width, n):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("streams,width,n", [(1, 40, 3), (2, 64, 70), (3, 192, 9), (4, 4100, 2), (2, 5000, 3)])
+@pytest.mark.parametrize("streams,width,n", [(1, 40, 3), (2, 64, 70), (3, 192, 9), (4, 4100, 2), (2, 5000, 3),
+                                             (2, 4500, 130), (8, 1024, 8), (3, 17000, 2)])
 def test_streams_write_read_and_norm_in_one_pass(dtype, streams, width, n):
     g = torch.Generator().manual_seed(streams + width)
     x = _rnd(g, n + 1, streams * width, scale=3.0)
