@@ -435,7 +435,7 @@ def main(argv=None) -> int:
                     help="also write a JSON file with the raw timing samples, their median and quartiles, the "
                          "commit and the software and device that ran them")
     ap.add_argument("--prefill-requests", type=int, default=2,
-                    help="prompts of 1,024 tokens in the prefill step (the contract's 2,048 tokens are 2)")
+                    help="prompts of 1,024 tokens in the prefill step (the default run's 2,048 tokens are 2)")
     ap.add_argument("--compare", choices=["viperax"], default=None,
                     help="prefill and decode of that design beside the GPT-2-style model at equal sizes (COMPARE_SIZES)")
     ap.add_argument("--prefill-only", action="store_true",

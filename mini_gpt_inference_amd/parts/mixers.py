@@ -8,7 +8,7 @@ import torch
 
 from ..ops import attention as attention_ops
 from ..ops import kernels, residual
-from ..ops.linear import LazyNorm, linear, linear_add, packed_weight, plain_residual
+from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, packed_weight, plain_residual
 from .base import (CacheBinding, KVNeed, MATRIX, Part, StateNeed, StepContext, VECTOR, WeightRequest,
                    register_mixer)
 from .positions import PositionEncoding
@@ -157,6 +157,10 @@ class LatentAttention(Mixer):
 
     graph_safe = True
     plan_safe = True
+    # up to this many rows queries, gate and latent come from one product with the matrices stacked
+    # (one launch less in a decode step); beyond it from two
+    JOINT_PRODUCT_MAX_ROWS = 128
+    JOINT_PRODUCT_MAX_WORK = 4 << 20     # rows x (query + gate columns); a smaller product has no full round to lose
 
     def __init__(self, width: int, n_head: int, head_dim: int, value_dim: int, rank: int, scale: float,
                  window: int = 0, eps: float = 1e-6, makes_latent: bool = True) -> None:
@@ -211,7 +215,16 @@ class LatentAttention(Mixer):
         n, ws = ctx.n_rows, ctx.workspace
         fast = not ctx.exact
         z = ws.get("latent_in", n, self.in_weight.shape[0], ctx.dtype)
-        linear(ctx, h, self.in_weight, None, z, n)
+        split = self.q_width + self.g_width
+        if self.makes_latent and n > self.JOINT_PRODUCT_MAX_ROWS and n * split > self.JOINT_PRODUCT_MAX_WORK:
+            # many rows: the few latent columns on top of queries and gate would start another
+            # round of the tiled kernel's tiles (17 x 16 tiles of 128 x 256 on 256 compute units
+            # where 16 x 16 fit), so the latent gets a small product of its own
+            hn = as_tensor(ctx, h)
+            linear(ctx, hn, self.in_weight[:split], None, z[:, :split], n)
+            linear(ctx, hn, self.in_weight[split:], None, z[:, split:], n)
+        else:
+            linear(ctx, h, self.in_weight, None, z, n)
         group = ctx.groups[binding.group]
         pool = group.k_pools[binding.index]
         if self.makes_latent:
