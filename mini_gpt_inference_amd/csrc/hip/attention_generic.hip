@@ -63,7 +63,7 @@ extern "C" int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int
   return mgpt_last_error();
 }
 
-#define MAX_DPL 4  // head_dim <= 256
+#define MAX_DPL 8  // head_dim <= 512
 
 template <typename T, bool FAST_EXP>
 __global__ __launch_bounds__(64) void paged_attention_generic_kernel(

@@ -204,9 +204,7 @@ def model_spec(cfg: ViperaxConfig) -> ModelSpec:
             feed_forward = PartSpec("table_experts", {"width": w, "hidden": f.ff, "n_experts": f.experts, "top": f.top,
                                                       "vocab_size": cfg.vocab, "shared_hidden": f.shared_ff}, names)
         if cfg.streams is None:
-            if feed_forward is None:
-                raise ConfigError(f"layer {i}: a layer without a feed-forward needs the hyper-connection arrangement")
-            arrangement = PartSpec("pre_norm", {"width": w})
+            arrangement = PartSpec("pre_norm" if feed_forward is not None else "pre_norm_mixer", {"width": w})
         else:
             hc = {}
             for q in ("1", "2") if feed_forward is not None else ("1",):

@@ -205,7 +205,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
     sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h."""
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
-    _need(head_dim <= 256, f"head size {head_dim} exceeds the kernel's limit of 256")
+    _need(head_dim <= 512, f"head size {head_dim} exceeds the kernel's limit of 512")
     _need_sinks(sinks, n_head)
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),

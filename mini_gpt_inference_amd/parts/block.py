@@ -55,6 +55,25 @@ class PreNorm(Arrangement):
         feed_forward.forward_add(ctx, LazyNorm(norm2, x, n), x)
 
 
+@register_arrangement("pre_norm_mixer")
+class PreNormMixerOnly(Arrangement):
+    """x = x + mixer(norm1(x)): a pre-norm layer that has no feed-forward."""
+
+    graph_safe = True
+    plan_safe = True
+    takes_pending_residual = True
+    roles = ("norm1", "mixer")
+
+    def __init__(self, width: int) -> None:
+        self.width = int(width)
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        mixer = parts["mixer"]
+        if not mixer.takes_pending_residual:
+            residual.settle(ctx, x, ctx.n_rows)
+        mixer.forward_add(ctx, LazyNorm(parts["norm1"], x, ctx.n_rows), x, bindings["mixer"], position)
+
+
 def flush_streams(ctx: StepContext, x: torch.Tensor, streams: int) -> None:
     """Makes the write into the residual streams that a sublayer has left pending, if any."""
     if ctx.pending_streams is not None:

@@ -168,8 +168,8 @@ class LatentAttention(Mixer):
         self.value_dim, self.rank = int(value_dim), int(rank)
         self.scale, self.window, self.eps = float(scale), int(window), float(eps)
         self.makes_latent = bool(makes_latent)
-        if not 0 < self.rank <= 256:
-            raise ValueError(f"latent size {self.rank}: the attention kernels take up to 256")
+        if not 0 < self.rank <= 512:
+            raise ValueError(f"latent size {self.rank}: the attention kernels take up to 512")
         self.q_width, self.g_width = self.n_head * self.head_dim, self.n_head * self.value_dim
         self.in_weight = self.uk_folded = self.uv_heads = None
 

@@ -57,11 +57,13 @@ RAW: Dict[str, dict] = {
                      _layer(_mixer(3, 8, 24, 40, 0.35, window=5), {"kind": "dense", "ff": 20}),
                      _layer(_mixer(1, 24, 8, 40, 0.2, window=3, kv_from=1), {"kind": "dense", "ff": 36})]},
     # no hyper-connections at all (no `streams` key), no masks, a latent of 64, three streams' worth of
-    # nothing: the plain pre-norm residual; top 3 of 4 with a shared expert
+    # nothing: the plain pre-norm residual; top 3 of 4 with a shared expert; a last layer without a
+    # feed-forward whose latent (320) is beyond what the bfloat16 attention kernels take
     "R": {"architecture": "Viperax", "vocab": 203, "width": 96, "norm": {"eps": 1e-4},
           "embedding": {"scale": 3.0}, "logit_scale": 1.0, "logit_softcap": 30.0,
           "layers": [_layer(_mixer(3, 32, 16, 64, 0.18), _moe(40, 4, 3, shared=24)),
-                     _layer(_mixer(2, 16, 48, 64, 0.25, kv_from=0), {"kind": "dense", "ff": 112})]},
+                     _layer(_mixer(2, 16, 48, 64, 0.25, kv_from=0), {"kind": "dense", "ff": 112}),
+                     _layer(_mixer(1, 40, 8, 320, 0.2, window=11), None)]},
     # three streams, a latent of 24 (the general kernel only), windows longer than most prompts
     "S": {"architecture": "Viperax", "vocab": 59, "width": 40, "streams": 3, "norm": {"eps": 1e-5},
           "embedding": {"scale": 6.0}, "logit_scale": 0.25, "logit_softcap": 5.0,
