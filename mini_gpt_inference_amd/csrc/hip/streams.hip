@@ -137,15 +137,13 @@ __global__ __launch_bounds__(T) void streams_step_kernel(
     int fold, int clear, const float* __restrict__ coef, float* __restrict__ u, const float* __restrict__ gain,
     const float* __restrict__ beta, float eps, OT* __restrict__ h, int width, int streams) {
   __shared__ float red[T / 64];
-  __shared__ float m_s[MGPT_MAX_STREAMS * MGPT_MAX_STREAMS], o_s[MGPT_MAX_STREAMS], c_s[MGPT_MAX_STREAMS];
   const int tid = threadIdx.x;
   const long n = blockIdx.x;
-  if (tid < streams * streams) m_s[tid] = fold ? mix[tid] : 0.f;
-  if (tid < streams) {
-    o_s[tid] = fold ? out[tid] : 0.f;
-    c_s[tid] = coef[tid];
-  }
-  __syncthreads();
+  // the coefficients are the same for every thread: read where they are used, they come through the
+  // scalar cache together with the first round of loads (no staging in LDS, no barrier before it)
+  const float* m_s = mix;
+  const float* o_s = out;
+  const float* c_s = coef;
   float* xr = x + n * (long)streams * width;
   // column c of the token, from its old streams and y: the streams rewritten (if a write is pending),
   // y cleared, u returned
@@ -175,9 +173,10 @@ __global__ __launch_bounds__(T) void streams_step_kernel(
     for (int s = 0; s < MGPT_MAX_STREAMS; ++s) old[s] = s < streams ? xr[(long)s * width + c] : 0.f;
     yv = fold ? y[n * width + c] : 0.f;
   };
-  float keep[SS_KEEP];
+  float keep[SS_KEEP], gk[SS_KEEP], bk[SS_KEEP];
   float sum = 0.f;
-  // four columns at a time: all their loads are asked for before the first of them is waited for
+  // four columns at a time: all their loads are asked for before the first of them is waited for,
+  // the gain and bias that the last pass needs among them
 #pragma unroll
   for (int i0 = 0; i0 < SS_KEEP; i0 += 4) {
     float old[4][MGPT_MAX_STREAMS], yv[4];
@@ -185,6 +184,8 @@ __global__ __launch_bounds__(T) void streams_step_kernel(
     for (int j = 0; j < 4; ++j) {
       const int c = tid + (i0 + j) * T;
       load(c < width ? c : 0, old[j], yv[j]);
+      gk[i0 + j] = gain[c < width ? c : 0];
+      bk[i0 + j] = beta ? beta[c < width ? c : 0] : 0.f;
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -218,11 +219,7 @@ __global__ __launch_bounds__(T) void streams_step_kernel(
 #pragma unroll
   for (int i = 0; i < SS_KEEP; ++i) {
     const int c = tid + i * T;
-    if (c < width) {
-      float v = (keep[i] - corr) * rstd * gain[c];
-      if (beta) v += beta[c];
-      h[n * width + c] = from_float<OT>(v);
-    }
+    if (c < width) h[n * width + c] = from_float<OT>((keep[i] - corr) * rstd * gk[i] + bk[i]);
   }
   for (int c = tid + SS_KEEP * T; c < width; c += T) {
     float v = ((u[n * width + c] - mean) - corr) * rstd * gain[c];

@@ -188,6 +188,7 @@ class DecoderModel:
             if run.reads_cache_of is not None and not (0 <= run.reads_cache_of < i):
                 raise ValueError(f"run {i} can only read the cache of an earlier run, not {run.reads_cache_of}")
         self.cache_layout = self._plan_cache()
+        self._stream_ones = None
 
     # ------------------------------------------------------------------ weights
     def _named_parts(self) -> List[Tuple[Part, PartSpec]]:
@@ -215,6 +216,10 @@ class DecoderModel:
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         self._bound = {name: tensors[name] for name in self.weight_requests()}
+        first = next(iter(tensors.values()), None)
+        # the coefficients of the plain sum of the streams, for the kernel that reads them weighted
+        self._stream_ones = (torch.ones(self.spec.streams, dtype=torch.float32, device=first.device)
+                             if first is not None and first.is_cuda else None)
         for part, spec in self._named_parts():
             replaced = part.bind({local: tensors[spec.weights[local]] for local in part.weight_requests()})
             for local, view in (replaced or {}).items():
@@ -362,21 +367,33 @@ class DecoderModel:
             if not layer.arrangement.takes_pending_residual:
                 residual.settle(ctx, x, n)
             layer.arrangement.run(ctx, x, layer.parts, bindings, self.position)
+        m = ctx.m_rows
+        # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
+        # whatever the vocabulary's size (50257 is odd)
+        vocab = self.spec.vocab_size
+        logits = ws.get("logits", m, -(-vocab // 4) * 4, torch.float32)[:, :vocab]
+        # every token's logits wanted, in order (the host has looked at the list): row i of the
+        # logits is token i, and the norm need not wait for the list before it can send for its rows
+        in_order = ctx.decode_only and m == n and ctx.logit_rows_in_order
+        if (ctx.pending_streams is not None and in_order and m and getattr(self.final_norm, "fusable_layer_norm", False)
+                and self._stream_ones is not None):
+            # the last sublayer's write into the streams, their sum and the final norm in one kernel
+            total = ws.get("residual_sum", n, self.spec.width, torch.float32)
+            normed = ws.get("final_normed", n, self.spec.width, ctx.dtype)
+            kernels.streams_step(x, ctx.pending_streams, self._stream_ones, total, self.final_norm.weight,
+                                 self.final_norm.bias, self.final_norm.eps, normed, n, streams)
+            ctx.pending_streams = None
+            self.head.forward(ctx, normed, logits, m)
+            ctx.pending = None
+            return logits[:m]
         _block.flush_streams(ctx, x, streams)
         if streams > 1:
             # the streams' sum is what the final norm reads
             total = ws.get("residual_sum", n, self.spec.width, torch.float32)
             kernels.streams_read(x, None, total, n, streams)
             x = total
-        m = ctx.m_rows
-        # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
-        # whatever the vocabulary's size (50257 is odd)
-        vocab = self.spec.vocab_size
-        logits = ws.get("logits", m, -(-vocab // 4) * 4, torch.float32)[:, :vocab]
         if m:
-            # every token's logits wanted, in order (the host has looked at the list): row i of the
-            # logits is token i, and the norm need not wait for the list before it can send for its rows
-            rows = None if ctx.decode_only and m == n and ctx.logit_rows_in_order else ctx.logit_rows
+            rows = None if in_order else ctx.logit_rows
             self.head.forward(ctx, LazyNorm(self.final_norm, x, m, rows=rows, buffer="final_normed"), logits, m)
         ctx.pending = None
         return logits[:m]
