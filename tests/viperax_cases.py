@@ -56,8 +56,8 @@ RAW: Dict[str, dict] = {
           "layers": [_layer(_mixer(1, 24, 8, 40, 0.2, window=1), _moe(32, 2, 1)),
                      _layer(_mixer(3, 8, 24, 40, 0.35, window=5), {"kind": "dense", "ff": 20}),
                      _layer(_mixer(1, 24, 8, 40, 0.2, window=3, kv_from=1), {"kind": "dense", "ff": 36})]},
-    # no hyper-connections at all (no `streams` key), no masks, a latent of 64, three streams' worth of
-    # nothing: the plain pre-norm residual; top 3 of 4 with a shared expert; a last layer without a
+    # no hyper-connections at all (no `streams` key: the plain pre-norm residual), no masks on the
+    # first two layers, a latent of 64; top 3 of 4 with a shared expert; a last layer without a
     # feed-forward whose latent (320) is beyond what the bfloat16 attention kernels take
     "R": {"architecture": "Viperax", "vocab": 203, "width": 96, "norm": {"eps": 1e-4},
           "embedding": {"scale": 3.0}, "logit_scale": 1.0, "logit_softcap": 30.0,
