@@ -4,6 +4,7 @@ just inside and just outside a window, for prompt portions and for single tokens
 against token-by-token decoding, portions down to two tokens and mixed batches with pages and
 request slots used again, in 32-bit and bfloat16; greedy generation through LLMEngine."""
 
+import json
 import math
 
 import numpy as np
@@ -381,6 +382,35 @@ def test_every_way_of_cutting_matches_the_plain_implementation(tmp_path_factory,
             _assert_within_rounding(folder, name, rid, reqs[rid], got[rid], want[rid], f"{name} {way} {rid}")
     assert replayer.cache.check() == 0 and not replayer.live
     assert all(replayer.cache.num_free_pages(g) == replayer.num_pages for g in range(len(replayer.cache.groups)))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_configurations(tmp_path, seed):
+    """Configurations drawn at random (tests/viperax_cases.py: random_raw), five requests of lengths
+    1 to 200 each, whole, in portions and mixed, in both dtypes.  bfloat16: a position may be one and
+    a half times over three times what rounding alone does, the mean may not."""
+    rng = np.random.default_rng(1000 + seed)
+    raw = cases.random_raw(rng)
+    folder = cases.write_raw_model(str(tmp_path / "m"), raw, seed)
+    cfg, w = V.read_model_folder(folder)
+    lens = [int(x) for x in rng.choice([1, 2, 5, 17, 33, 64, 70, 97, 130, 200], size=5)]
+    reqs = {f"r{i}": helpers.random_ids(rng, raw["vocab"], n) for i, n in enumerate(lens)}
+    want = {rid: V.forward(cfg, w, ids)[0].numpy() for rid, ids in reqs.items()}
+    noise = {rid: _row_errors(_rounded_twin(cfg, w, ids), want[rid]) for rid, ids in reqs.items()}
+    for dtype in ("float32", "bfloat16"):
+        for way in ("whole", "portions", "mixed"):
+            plan = helpers.PLANS[way](reqs, np.random.default_rng(5))
+            replayer = TraceReplayer(folder, dtype, plan.tight_tokens(16), page_size=16, max_live=4, poison=True)
+            got = plan.assemble(helpers.run_plan_in_process(replayer, plan), {r: len(t) for r, t in reqs.items()},
+                                raw["vocab"])
+            for rid in reqs:
+                what = f"seed {seed} {dtype} {way} {rid} ({json.dumps(raw)})"
+                if dtype == "float32":
+                    helpers.assert_close(got[rid], want[rid], dtype, what)
+                    continue
+                assert np.isfinite(got[rid]).all(), what
+                err = _row_errors(got[rid], want[rid])
+                assert err.max() <= 4.5 * noise[rid].max() and err.mean() <= 3.0 * noise[rid].mean(), what
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -91,3 +91,56 @@ def write_model(path: str, name: str, edit: Optional[Callable[[Dict[str, torch.T
     write_config_json(path, cfg)
     save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(path, "model.safetensors"))
     return path
+
+
+def random_raw(rng) -> dict:
+    """A random config.json: widths, layer counts, streams (none to 4), heads 1 to 5, query/key and
+    value sizes that are no multiples of 16, latents from 16 to 160 (some layers reading an earlier
+    layer's of the same size), windows from 1 to longer than the prompts or none, every kind of
+    feed-forward or none."""
+    width = int(rng.choice([40, 64, 72, 96, 136, 200, 256]))
+    streams = rng.choice([None, 1, 2, 3, 4])
+    rank_all = int(rng.choice([16, 24, 40, 48, 64, 80, 96, 128, 160]))
+    layers, own = [], []
+    for i in range(int(rng.integers(2, 6))):
+        dim = int(rng.choice([8, 12, 16, 24, 32, 40, 64]))
+        rank = rank_all if rng.random() < 0.7 else int(rng.choice([16, 32, 56]))
+        mixer = _mixer(int(rng.integers(1, 6)), dim, int(rng.choice([8, 16, 20, 32, 48])), rank,
+                       float(rng.choice([0.1, 0.25, dim ** -0.5])),
+                       window=int(rng.choice([1, 2, 7, 16, 17, 33, 64, 100])) if rng.random() < 0.8 else None)
+        sources = [j for j in own if layers[j]["mixer"]["kv_rank"] == rank]
+        if sources and rng.random() < 0.5:
+            mixer["kv_from"] = int(rng.choice(sources))
+        else:
+            own.append(i)
+        kind = rng.choice(["none", "dense", "moe"])
+        if kind == "none":
+            mlp = None
+        elif kind == "dense":
+            mlp = {"kind": "dense", "ff": int(rng.choice([24, 40, 100, 128]))}
+        else:
+            experts = int(rng.integers(2, 10))
+            mlp = _moe(int(rng.choice([8, 24, 32, 48])), experts, int(rng.integers(1, min(experts, 3) + 1)),
+                       shared=int(rng.choice([16, 40, 64])) if rng.random() < 0.5 else None)
+        layers.append(_layer(mixer, mlp))
+    raw = {"architecture": "Viperax", "vocab": int(rng.choice([50, 131, 300, 577])), "width": width,
+           "norm": {"eps": float(rng.choice([1e-6, 1e-5]))},
+           "embedding": {"scale": float(rng.choice([1.0, 4.0, width ** 0.5]))},
+           "logit_scale": float(rng.choice([0.25, 1.0])), "layers": layers}
+    if streams is not None:
+        raw["streams"] = int(streams)
+    if rng.random() < 0.7:
+        raw["logit_softcap"] = float(rng.choice([5.0, 15.0, 30.0]))
+    return raw
+
+
+def write_raw_model(path: str, raw: dict, seed: int, std_scale: float = 1.5) -> str:
+    cfg = viperax.config_from_json(raw)
+    tensors = random_tensors(cfg, seed, torch.bfloat16, std_scale)
+    for key in tensors:
+        if key.endswith(".sink"):
+            tensors[key] = (tensors[key].float() * 2.0 + 1.0).to(torch.bfloat16)
+    os.makedirs(path, exist_ok=True)
+    write_config_json(path, cfg)
+    save_file({k: v.contiguous() for k, v in tensors.items()}, os.path.join(path, "model.safetensors"))
+    return path
