@@ -24,8 +24,22 @@ class KVStore:
             # a joint group's pages hold one tensor that is both keys and values
             shape = (spec.n_pools, 1 if spec.joint else 2, geo.num_pages, spec.n_kv_head, geo.page_size, spec.head_dim)
             self.pools.append(torch.full(shape, fill, dtype=dtype, device=device))
-        self.state_pools = [torch.zeros((max_requests, n), dtype=torch.float32, device=device)
+        self.state_pools = [torch.full((max_requests, n), fill, dtype=torch.float32, device=device)
                             for n in layout.state_numels]
+
+    def snapshot_states(self, slots: Sequence[int]) -> List[torch.Tensor]:
+        """Copies of the given requests' rows of every state pool.  Pages take a step's keys and values
+        a second time without harm; a state that the step has advanced must not be advanced again, so
+        whoever runs a step's forward pass twice puts these back in between (restore_states)."""
+        if not self.state_pools or not len(slots):
+            return []
+        index = torch.tensor(list(slots), dtype=torch.long, device=self.state_pools[0].device)
+        return [index] + [pool.index_select(0, index) for pool in self.state_pools]
+
+    def restore_states(self, saved: List[torch.Tensor]) -> None:
+        if saved:
+            for pool, rows in zip(self.state_pools, saved[1:]):
+                pool.index_copy_(0, saved[0], rows)
 
     def k_pools(self, group: int) -> List[torch.Tensor]:
         p = self.pools[group]

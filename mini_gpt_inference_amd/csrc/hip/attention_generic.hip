@@ -9,7 +9,8 @@
 // attention: S = q k^T * scale; a query at absolute position p sees the keys at
 // positions max(0, p-window+1)..p of its own request (window 0 = all of them);
 // softmax over keys in 32-bit (with `sinks`, one more term exp(sinks[head]) in its denominator that
-// has no value); y = P v (reference: src/minigpt_infer/model.py:61-87,
+// has no value; with `softcap` > 0 every score becomes softcap * tanh(score / softcap) first);
+// y = P v (reference: src/minigpt_infer/model.py:61-87,
 // the rule col <= cache_len + row of src/minigpt_infer/batch.py:202-227).
 //
 // The general kernel runs one wave per (token, head).  Keys are reduced in
@@ -71,7 +72,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ cu_q, const int* __restrict__ seq_lens, const int* __restrict__ q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* __restrict__ sinks) {
+    const float* __restrict__ sinks, float softcap) {
   __shared__ float q_s[MAX_DPL * MGPT_WAVE];
   __shared__ float p_s[MGPT_WAVE];
   __shared__ int page_s[MGPT_WAVE];
@@ -109,6 +110,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(q_s[d], to_float<T>(kr[d]), dot);
       s = dot * scale;
+      if (softcap > 0.f) s = softcap * tanhf(s / softcap);
     }
     const float m_new = fmaxf(m, wave_max(s));
     float p = 0.f;
@@ -160,7 +162,7 @@ extern "C" int mgpt_paged_attention_generic(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int dtype, int fast_exp, const float* sinks, hipStream_t stream) {
+    int dtype, int fast_exp, const float* sinks, float softcap, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
@@ -171,7 +173,7 @@ extern "C" int mgpt_paged_attention_generic(
 #define LAUNCH(T, F)                                                                              \
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, F>), grid, block, 0, stream, (const T*)q, ldq, \
                      (T*)out, ldo, (const T*)kpool, (const T*)vpool, block_tables, max_blocks, cu_q,  \
-                     seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim, page_size, scale, window, sinks)
+                     seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim, page_size, scale, window, sinks, softcap)
   if (dtype == MGPT_F32) {
     if (fast_exp) LAUNCH(float, true); else LAUNCH(float, false);
   } else if (dtype == MGPT_BF16) {

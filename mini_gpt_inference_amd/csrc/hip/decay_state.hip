@@ -1,0 +1,158 @@
+// Linear attention with a fixed decay per head: a mixer whose memory is one float32 matrix per
+// request and head instead of a cache of keys and values.
+//
+//   S_t = decay_h S_(t-1) + k_t v_t^T      (S: [D, E], zero before a request's first token)
+//   o_t = S_t^T q_t
+//
+// q, k [H, D] and v [H, E] of a token lie in one row of `z` (the output of the stacked projection),
+// in the compute dtype.  On their way in they may pass an activation (silu), q and k a rotation by
+// position (pairs (i, i + rot_dims/2), angle position * freq[i], all float32), and k a constant
+// scale.  Everything from there on is float32: the state, its decay, the products that enter it and
+// the output.  On the way out a head's output may be divided by its root mean square (eps inside
+// the root) and multiplied by silu(gate); the result is stored as float32 or in the compute dtype.
+//
+// One workgroup per (request, head) walks the request's tokens of this step in order, whatever
+// their number (a prompt, a portion of one, one decoded token), from the state that the step
+// before left in the request's slot, and leaves the new state there.  The state lives in
+// registers: thread (dg, e) owns S[d][e] for d = dg, dg + NG, ...; the tokens' q, k, v are staged
+// through LDS eight at a time, and the partial sums over dg meet there once per eight tokens.
+#include "common.h"
+#include "dtype_io.h"
+#include "launchers.h"
+
+#define DS_MAX 256  // largest D and E
+#define DS_TC 8     // tokens staged at once
+
+__device__ __forceinline__ float ds_act(float v, int act) { return act == 1 ? v / (1.0f + expf(-v)) : v; }
+
+template <int R>
+__global__ __launch_bounds__(256) void decay_state_kernel(
+    const void* __restrict__ z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head, int D, int E,
+    int act, const int* __restrict__ positions, const float* __restrict__ freq, int rot_dims, float k_scale,
+    const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ state_slots,
+    const int* __restrict__ cu_q, float norm_eps, void* __restrict__ out, int out_dtype, long ldo) {
+  __shared__ float q_s[DS_TC][DS_MAX], k_s[DS_TC][DS_MAX], v_s[DS_TC][DS_MAX], red[DS_TC][256];
+  const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
+  const int slot = state_slots[r];
+  const int t_begin = cu_q[r], t_end = cu_q[r + 1];
+  if (slot < 0 || t_end <= t_begin) return;     // a request of the padding
+  const int NG = 256 / E < D ? 256 / E : D;     // groups of threads over d (at least 1: E <= 256)
+  const bool owner = tid < NG * E;
+  const int e = tid % E, dg = tid / E;
+  const int count = owner ? (D - dg + NG - 1) / NG : 0;
+  const float lambda = decay[h];
+  float S[R];
+  float* st = state + ((long)slot * n_head + h) * (long)D * E;
+  const bool fresh = positions[t_begin] == 0;   // the request's first token: its state starts at zero
+#pragma unroll
+  for (int j = 0; j < R; ++j) S[j] = (j < count && !fresh) ? st[(long)(dg + j * NG) * E + e] : 0.f;
+  const int half = rot_dims / 2;
+  const int wave = tid >> 6, lane = tid & 63;
+
+  for (int t0 = t_begin; t0 < t_end; t0 += DS_TC) {
+    const int nt = t_end - t0 < DS_TC ? t_end - t0 : DS_TC;
+    __syncthreads();     // the chunk before is read
+    for (int i = tid; i < nt * D; i += 256) {
+      const int tt = i / D, d = i - tt * D;
+      const long row = (long)(t0 + tt) * ldz + (long)h * D + d;
+      q_s[tt][d] = ds_act(load_f(z, dtype, row + q_off), act);
+      k_s[tt][d] = ds_act(load_f(z, dtype, row + k_off), act);
+    }
+    for (int i = tid; i < nt * E; i += 256) {
+      const int tt = i / E, c = i - tt * E;
+      v_s[tt][c] = ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + c), act);
+    }
+    __syncthreads();
+    if (freq) {
+      for (int i = tid; i < nt * half; i += 256) {
+        const int tt = i / half, c = i - tt * half;
+        const float a = (float)positions[t0 + tt] * freq[c];
+        const float co = cosf(a), si = sinf(a);
+        const float qu = q_s[tt][c], qw = q_s[tt][c + half], ku = k_s[tt][c], kw = k_s[tt][c + half];
+        q_s[tt][c] = qu * co - qw * si;
+        q_s[tt][c + half] = qw * co + qu * si;
+        k_s[tt][c] = (ku * co - kw * si) * k_scale;
+        k_s[tt][c + half] = (kw * co + ku * si) * k_scale;
+      }
+      if (k_scale != 1.0f)
+        for (int i = tid; i < nt * (D - rot_dims); i += 256) {
+          const int tt = i / (D - rot_dims), c = rot_dims + i - tt * (D - rot_dims);
+          k_s[tt][c] *= k_scale;
+        }
+    } else if (k_scale != 1.0f) {
+      for (int i = tid; i < nt * D; i += 256) k_s[i / D][i % D] *= k_scale;
+    }
+    __syncthreads();
+    if (owner) {
+      for (int tt = 0; tt < nt; ++tt) {
+        const float ve = v_s[tt][e];
+        float acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+          if (j < count) {
+            const int d = dg + j * NG;
+            S[j] = fmaf(lambda, S[j], k_s[tt][d] * ve);
+            acc = fmaf(S[j], q_s[tt][d], acc);
+          }
+        }
+        red[tt][tid] = acc;
+      }
+    }
+    __syncthreads();
+    // a wave a token: the sums over dg in order, the head's norm, the gate, the store
+    for (int tt = wave; tt < nt; tt += 4) {
+      float ss = 0.f;
+      for (int c = lane; c < E; c += 64) {
+        float o = 0.f;
+        for (int g = 0; g < NG; ++g) o += red[tt][g * E + c];
+        red[tt][c] = o;
+        ss = fmaf(o, o, ss);
+      }
+      float scale = 1.0f;
+      if (norm_eps >= 0.f) scale = 1.0f / sqrtf(wave_sum(ss) / (float)E + norm_eps);
+      const long n = t0 + tt;
+      for (int c = lane; c < E; c += 64) {
+        float o = red[tt][c] * scale;
+        if (g_off >= 0) {
+          const float g = load_f(z, dtype, n * ldz + g_off + (long)h * E + c);
+          o *= g / (1.0f + expf(-g));
+        }
+        store_f(out, out_dtype, n * ldo + (long)h * E + c, o);
+      }
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+    if (j < count) st[(long)(dg + j * NG) * E + e] = S[j];
+}
+
+// z: [n_tokens, ldz] rows in `dtype`; q at q_off, k at k_off, v at v_off, the gate at g_off (-1: none), head by head.
+// state: [slots, n_head * D * E] float32; state_slots[r] the slot of request r (-1: none), cu_q its tokens.
+extern "C" int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head,
+                                int head_dim, int value_dim, int act, const int* positions, const float* freq,
+                                int rot_dims, float k_scale, const float* decay, float* state, const int* state_slots,
+                                const int* cu_q, int n_req, float norm_eps, void* out, int out_dtype, long ldo,
+                                hipStream_t stream) {
+  if (n_req == 0) return MGPT_OK;
+  if (!z || !positions || !decay || !state || !state_slots || !cu_q || !out) return MGPT_ERR_NULL;
+  if (!dtype_ok(dtype) || !dtype_ok(out_dtype)) return MGPT_ERR_BAD_DTYPE;
+  const int D = head_dim, E = value_dim;
+  if (n_req < 0 || n_head <= 0 || D <= 0 || E <= 0 || D > DS_MAX || E > DS_MAX || rot_dims < 0 || (rot_dims & 1) ||
+      rot_dims > D || (act != 0 && act != 1))
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
+  const int ng = 256 / E < D ? 256 / E : D;
+  const int per_thread = (D + ng - 1) / ng;
+  dim3 grid(n_req, n_head), block(256);
+#define DS_LAUNCH(R)                                                                                                   \
+  hipLaunchKernelGGL(decay_state_kernel<R>, grid, block, 0, stream, z, dtype, ldz, q_off, k_off, v_off, g_off, n_head, D, E, \
+                     act, positions, rot_dims ? freq : nullptr, rot_dims, k_scale, decay, state, state_slots, cu_q, norm_eps, \
+                     out, out_dtype, ldo)
+  if (per_thread <= 8) DS_LAUNCH(8);
+  else if (per_thread <= 32) DS_LAUNCH(32);
+  else if (per_thread <= 64) DS_LAUNCH(64);
+  else if (per_thread <= 128) DS_LAUNCH(128);
+  else return MGPT_ERR_BAD_SHAPE;     // a state of more than 128 values a thread
+#undef DS_LAUNCH
+  return mgpt_last_error();
+}

@@ -19,27 +19,30 @@
 
 template <typename T, bool FAST>
 __global__ void gated_unit_kernel(const T* __restrict__ z, long ldz, T* __restrict__ act, long lda, long total,
-                                  int hidden) {
+                                  int hidden, int kind) {
   const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
   if (i >= total) return;
   const long n = i / hidden;
   const int j = (int)(i - n * hidden);
   const float g = to_float<T>(z[n * ldz + j]), u = to_float<T>(z[n * ldz + hidden + j]);
-  const float s = FAST ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) : g / (1.0f + expf(-g));
+  float s;
+  if (kind == 1) s = fmaxf(g, 0.f);                                  // relu
+  else if (kind == 2) s = FAST ? gelu_tanh_fast(g) : gelu_tanh(g);
+  else s = FAST ? g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) : g / (1.0f + expf(-g));   // silu
   act[n * lda + j] = from_float<T>(s * u);
 }
 
 extern "C" int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype,
-                               int fast, hipStream_t stream) {
+                               int fast, int kind, hipStream_t stream) {
   if (n_rows == 0) return MGPT_OK;
   if (!z || !act) return MGPT_ERR_NULL;
-  if (n_rows < 0 || hidden <= 0 || ldz < 2L * hidden || lda < hidden) return MGPT_ERR_BAD_SHAPE;
+  if (n_rows < 0 || hidden <= 0 || ldz < 2L * hidden || lda < hidden || kind < 0 || kind > 2) return MGPT_ERR_BAD_SHAPE;
   const long total = (long)n_rows * hidden;
   const long blocks = (total + 255) / 256;
   if (blocks > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
   dim3 grid((unsigned)blocks), block(256);
 #define GU_LAUNCH(T, F) \
-  hipLaunchKernelGGL((gated_unit_kernel<T, F>), grid, block, 0, stream, (const T*)z, ldz, (T*)act, lda, total, hidden)
+  hipLaunchKernelGGL((gated_unit_kernel<T, F>), grid, block, 0, stream, (const T*)z, ldz, (T*)act, lda, total, hidden, kind)
   if (dtype == MGPT_F32) {
     if (fast) GU_LAUNCH(float, true); else GU_LAUNCH(float, false);
   } else if (dtype == MGPT_BF16) {

@@ -28,7 +28,7 @@ int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, voi
 int mgpt_paged_attention_generic(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int dtype,
-    int fast_exp, const float* sinks, hipStream_t stream);
+    int fast_exp, const float* sinks, float softcap, hipStream_t stream);
 // attention_prefill.hip
 int mgpt_prefill_attention_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req, int
@@ -131,7 +131,7 @@ int mgpt_heads_linear_mfma(const void* a, long lda, const void* w, void* out, lo
     int n_rows, int n_head, int n_out, int k_dim, hipStream_t stream);
 // experts.hip
 int mgpt_gated_unit(const void* z, long ldz, void* act, long lda, int n_rows, int hidden, int dtype, int fast,
-    hipStream_t stream);
+    int kind, hipStream_t stream);
 int mgpt_expert_route(const int* ids, const int* q_req, const int* table, int top, int n_rows, int n_experts,
     int* slot_token, int* slot_pair, int* pair_slot, int* tile_expert, int n_slots, int n_tiles, int tile_rows,
     hipStream_t stream);
@@ -145,6 +145,26 @@ int mgpt_grouped_linear_mfma(const void* a, long lda, const int* a_rows, const v
     int n_out, int k_dim, hipStream_t stream);
 int mgpt_expert_combine(const float* pair_out, const int* pair_slot, const int* q_req, float* y, int n_rows, int
     width, int top, float weight, hipStream_t stream);
+// rms_norm.hip
+int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* rows, const float* gain, float offset, float eps,
+    float mult, const void* gate, int gate_dtype, long ldg, int gate_act, void* out, int out_dtype, long ldo,
+    int accumulate, float* zero, long ldz, int zero_width, int n_rows, int groups, int x_gstride, int o_gstride,
+    int width, hipStream_t stream);
+int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, const float* g0, const float* g1, const float* g2,
+    const float* g3, int n_branches, float coef, float* x, const float* gain_post, float offset, float eps, float mult,
+    const float* gain_next, void* h, int h_dtype, int n_rows, int width, hipStream_t stream);
+// qk_prepare.hip
+int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head, int n_kv_head,
+    int head_dim, int value_dim, int head_stride, const int* positions, const float* freq, int rot_dims, float norm_eps,
+    const float* mix_lambda, void* v_other, long ld_other, int mix_mode, void* kpool, void* vpool,
+    const int* slot_mapping, int page_size, int n_tokens, hipStream_t stream);
+int mgpt_head_gate(void* y, int dtype, long ldy, int head_stride, int width, const void* gate, int gate_dtype,
+    long ldg, int n_rows, int n_head, hipStream_t stream);
+// decay_state.hip
+int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head,
+    int head_dim, int value_dim, int act, const int* positions, const float* freq, int rot_dims, float k_scale,
+    const float* decay, float* state, const int* state_slots, const int* cu_q, int n_req, float norm_eps, void* out,
+    int out_dtype, long ldo, hipStream_t stream);
 // linear_mfma.hip
 int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_stride, const int* row_expert, const
     int* row_valid, int group_rows, void* out, int out_dtype, long ldo, int n_rows, int n_out, int k_dim,
@@ -191,4 +211,9 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_grouped_linear) \
   X(mgpt_expert_combine) \
   X(mgpt_gather_rows) \
-  X(mgpt_linear_mfma_grouped)
+  X(mgpt_linear_mfma_grouped) \
+  X(mgpt_rms_norm) \
+  X(mgpt_rms_post_norm) \
+  X(mgpt_qk_prepare) \
+  X(mgpt_head_gate) \
+  X(mgpt_decay_state)

@@ -1,0 +1,159 @@
+// Root-mean-square norms over float32 statistics.
+//
+//   unit(x) = x / sqrt(mean(x^2) + eps)
+//
+// rms_norm: out = [out +] mult * unit(x) * (offset + gain) [* act(gate)], per segment: a row holds
+// `groups` segments of `width` values (one for a norm over the row, one per head for a norm per
+// head).  gain may be absent (a norm without a weight), offset is 1 for a gain stored as its
+// distance from one.  Rows may be gathered (`rows`), and a second buffer may be cleared on the way
+// (the buffer the next sublayer adds its output into).
+//
+// rms_post_norm: the step between two sublayers of a layer whose sublayers are normed on both
+// sides, one workgroup a row:
+//   y = sum_b coef * unit(y_b) * gain_b          (only with several branches; else y = y_0)
+//   x += mult * unit(y) * (offset + gain_post)
+//   h = unit(x) * (offset + gain_next)           (if there is a next norm)
+//   y_b = 0                                       (ready for the next sublayer's additions)
+// Sums of squares are taken in float32 in a fixed order (lane-strided, then across the wave, then
+// across the waves in order), so a row's result does not depend on the other rows of the step.
+#include "common.h"
+#include "dtype_io.h"
+#include "launchers.h"
+
+#define RMS_ACT_NONE 0
+#define RMS_ACT_SILU 1
+#define RMS_ACT_SIGMOID 2
+
+__device__ __forceinline__ float rms_gate_act(float g, int act) {
+  if (act == RMS_ACT_SILU) return g / (1.0f + expf(-g));
+  if (act == RMS_ACT_SIGMOID) return 1.0f / (1.0f + expf(-g));
+  return g;
+}
+
+// one wave per segment
+__global__ __launch_bounds__(256) void rms_norm_kernel(
+    const void* __restrict__ x, int x_dtype, long ldx, const int* __restrict__ rows,
+    const float* __restrict__ gain, float offset, float eps, float mult, const void* __restrict__ gate,
+    int gate_dtype, long ldg, int gate_act, void* out, int out_dtype, long ldo, int accumulate,
+    float* __restrict__ zero, long ldz, int zero_width, int n_rows, int groups, int x_gstride, int o_gstride,
+    int width) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const long seg = (long)blockIdx.x * 4 + wave;
+  if (seg >= (long)n_rows * groups) return;
+  const int row = (int)(seg / groups), g = (int)(seg - (long)row * groups);
+  const int src = rows ? rows[row] : row;
+  const long xb = (long)src * ldx + (long)g * x_gstride;
+  float ss = 0.f;
+  for (int c = lane; c < width; c += 64) {
+    const float v = load_f(x, x_dtype, xb + c);
+    ss = fmaf(v, v, ss);
+  }
+  ss = wave_sum(ss);
+  const float r = mult / sqrtf(ss / (float)width + eps);
+  const long ob = (long)row * ldo + (long)g * o_gstride;
+  const long gb = (long)row * ldg + (long)g * o_gstride;
+  for (int c = lane; c < width; c += 64) {
+    float v = load_f(x, x_dtype, xb + c) * r;
+    if (gain) v *= offset + gain[(long)g * width + c];
+    if (gate) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), gate_act);
+    if (accumulate) v += load_f(out, out_dtype, ob + c);
+    store_f(out, out_dtype, ob + c, v);
+  }
+  if (zero && g == 0)
+    for (int c = lane; c < zero_width; c += 64) zero[(long)row * ldz + c] = 0.f;
+}
+
+extern "C" int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* rows, const float* gain, float offset,
+                             float eps, float mult, const void* gate, int gate_dtype, long ldg, int gate_act,
+                             void* out, int out_dtype, long ldo, int accumulate, float* zero, long ldz,
+                             int zero_width, int n_rows, int groups, int x_gstride, int o_gstride, int width,
+                             hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!x || !out) return MGPT_ERR_NULL;
+  if (n_rows < 0 || groups <= 0 || width <= 0 || zero_width < 0) return MGPT_ERR_BAD_SHAPE;
+  if (!dtype_ok(x_dtype) || !dtype_ok(out_dtype) || (gate && !dtype_ok(gate_dtype))) return MGPT_ERR_BAD_DTYPE;
+  const long segs = (long)n_rows * groups;
+  if (segs > (1L << 32)) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)((segs + 3) / 4)), dim3(256), 0, stream, x, x_dtype, ldx, rows,
+                     gain, offset, eps, mult, gate, gate_dtype, ldg, gate_act, out, out_dtype, ldo, accumulate, zero,
+                     ldz, zero_width, n_rows, groups, x_gstride, o_gstride, width);
+  return mgpt_last_error();
+}
+
+// sum over the workgroup's 256 threads, the same value in every thread; waves are added in order
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();      // the scratch's readers of the call before are done
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  return (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+}
+
+#define RMS_MAX_BRANCHES 4
+
+struct RmsBranches {
+  float* y[RMS_MAX_BRANCHES];
+  const float* gain[RMS_MAX_BRANCHES];
+};
+
+__global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int n_branches, float coef, float* __restrict__ x,
+                                                            const float* __restrict__ gain_post, float offset, float eps,
+                                                            float mult, const float* __restrict__ gain_next,
+                                                            void* __restrict__ h, int h_dtype, int n_rows, int width) {
+  __shared__ float scratch[4];
+  const int row = blockIdx.x;
+  if (row >= n_rows) return;
+  const long base = (long)row * width;
+  float* y0 = br.y[0] + base;
+  if (n_branches > 1) {
+    // the branches' outputs, each normed with its own plain gain, averaged into the first one's buffer
+    float r[RMS_MAX_BRANCHES];
+    for (int b = 0; b < n_branches; ++b) {
+      const float* yb = br.y[b] + base;
+      float ss = 0.f;
+      for (int c = threadIdx.x; c < width; c += 256) ss = fmaf(yb[c], yb[c], ss);
+      r[b] = coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+    }
+    for (int c = threadIdx.x; c < width; c += 256) {
+      float v = 0.f;
+      for (int b = 0; b < n_branches; ++b) {
+        v = fmaf(br.y[b][base + c] * r[b], br.gain[b][c], v);
+        if (b) br.y[b][base + c] = 0.f;
+      }
+      y0[c] = v;      // read again below by the thread that wrote it
+    }
+  }
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) ss = fmaf(y0[c], y0[c], ss);
+  const float ry = mult / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+  float sx = 0.f;
+  for (int c = threadIdx.x; c < width; c += 256) {
+    const float v = x[base + c] + y0[c] * ry * (offset + gain_post[c]);
+    x[base + c] = v;
+    y0[c] = 0.f;
+    sx = fmaf(v, v, sx);
+  }
+  if (!gain_next) return;
+  const float rx = 1.0f / sqrtf(block_sum_256(sx, scratch) / (float)width + eps);
+  for (int c = threadIdx.x; c < width; c += 256)
+    store_f(h, h_dtype, base + c, x[base + c] * rx * (offset + gain_next[c]));
+}
+
+// y_ptrs / gain_ptrs: n_branches device pointers each (float32 [n_rows, width] buffers; [width] gains, unused
+// with one branch).  x, y: contiguous float32 rows.
+extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, const float* g0, const float* g1,
+                                  const float* g2, const float* g3, int n_branches, float coef, float* x,
+                                  const float* gain_post, float offset, float eps, float mult, const float* gain_next,
+                                  void* h, int h_dtype, int n_rows, int width, hipStream_t stream) {
+  if (n_rows == 0) return MGPT_OK;
+  if (!x || !y0 || !gain_post || (gain_next && !h)) return MGPT_ERR_NULL;
+  if (n_rows < 0 || width <= 0 || n_branches < 1 || n_branches > RMS_MAX_BRANCHES) return MGPT_ERR_BAD_SHAPE;
+  if (gain_next && !dtype_ok(h_dtype)) return MGPT_ERR_BAD_DTYPE;
+  RmsBranches br = {{y0, y1, y2, y3}, {g0, g1, g2, g3}};
+  for (int b = 0; b < n_branches; ++b)
+    if (!br.y[b] || (n_branches > 1 && !br.gain[b])) return MGPT_ERR_NULL;
+  hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, x, gain_post,
+                     offset, eps, mult, gain_next, h, h_dtype, n_rows, width);
+  return mgpt_last_error();
+}

@@ -108,11 +108,15 @@ class _GraphedDecode:
         if self.graph is None:
             # once eagerly, so that every workspace buffer and every derived copy of a matrix exists
             # before capture; then once more, counted and recorded: the step as every later one runs
+            # (a mixer's per-request state must see this step once: what the eager runs do to it is undone)
+            saved = self.runner.store.snapshot_states(shape.slots)
             self._launch(shape)
             torch.cuda.synchronize()
+            self.runner.store.restore_states(saved)
             self.workspace.frozen = True
             self.arena.upload()
             self._launch(shape, record=self.runner.plan_steps)
+            self.runner.store.restore_states(saved)
             torch.cuda.synchronize()
             self.graph = self._capture(shape, 1)
             # the eager launch above did this step's work and moved the device arrays on to the

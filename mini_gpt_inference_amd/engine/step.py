@@ -314,12 +314,28 @@ class ModelRunner:
             bucket.graph.replay()
             self.num_replayed_steps += 1
             return bucket.logits[:shape.n_logits]
+        capture_bucket = (exact.seen < self.CAPTURE_AT and bucket.seen >= self.CAPTURE_AT
+                          and not self._live(bucket, arena))
+        if capture_bucket:
+            self._warm_up(arena, shape, lead_cap)
         logits = self._planned_or_recorded(exact, arena, shape)
         if exact.seen >= self.CAPTURE_AT:
             self._capture(exact, arena, shape, None)
-        elif bucket.seen >= self.CAPTURE_AT and not self._live(bucket, arena):
+        elif capture_bucket:
             self._capture(bucket, arena, shape, lead_cap)
         return logits
+
+    def _warm_up(self, arena: StepArena, shape: StepShape, lead_cap: int) -> None:
+        """A bucket's graph runs over more rows than any eager step did, so the padded step runs once
+        eagerly before it is captured: every buffer it needs exists then.  It runs ahead of the step's
+        own pass and from the same state: what it does to the requests' state is undone, and what it
+        writes into the pages the step's own pass writes again, value for value.  (Behind that pass it
+        would start from a state that has this step's tokens in it already, and a layer above such a
+        mixer would store other keys and values.)"""
+        saved = self.store.snapshot_states(shape.slots)
+        with kernels.pinned_stream():
+            self.model.forward(self.context(arena, shape, padded=True, lead_cap=lead_cap))
+        self.store.restore_states(saved)
 
     def _plan_live(self, entry: _StepGraph, arena: StepArena) -> bool:
         return (entry.plan is not None and entry.plan_arena is arena
@@ -366,8 +382,7 @@ class ModelRunner:
 
     def _capture(self, entry: _StepGraph, arena: StepArena, shape: StepShape, lead_cap: Optional[int]) -> None:
         """Records the step that the arena holds for the next of its shape (lead_cap None) or of its
-        bucket.  A bucket's graph runs over more rows than the eager step before it did, so it runs
-        once eagerly first: every buffer it needs exists then."""
+        bucket (whose padded step has run once eagerly: _warm_up)."""
         def forward():
             with kernels.pinned_stream():
                 if lead_cap is None and self._plan_live(entry, arena):
@@ -377,8 +392,6 @@ class ModelRunner:
                 return self.model.forward(ctx)
         entry.graph = None
         self.num_graph_captures += 1
-        if lead_cap is not None:
-            forward()
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())

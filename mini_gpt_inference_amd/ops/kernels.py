@@ -200,9 +200,11 @@ def _check_attention_args(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, 
 def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                             block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                             q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
-                            window: int = 0, fast_exp: bool = False, sinks: Optional[torch.Tensor] = None) -> None:
+                            window: int = 0, fast_exp: bool = False, sinks: Optional[torch.Tensor] = None,
+                            softcap: float = 0.0) -> None:
     """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype).
-    sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h."""
+    sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h.
+    softcap > 0: every score becomes softcap * tanh(score / softcap) before the softmax."""
     n_kv_head, page_size, head_dim = _check_attention_args(
         q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head)
     _need(head_dim <= 512, f"head size {head_dim} exceeds the kernel's limit of 512")
@@ -210,7 +212,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), _stream())
+        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), float(softcap), _stream())
     _check(rc, "paged_attention_generic")
 
 
@@ -1079,14 +1081,19 @@ EXPERT_TILES = (16, 64, 256)
 MAX_EXPERTS = 1024
 
 
-def gated_unit(z: torch.Tensor, act: torch.Tensor, n_rows: int, hidden: int, fast: bool = False) -> None:
-    """act[n][j] = silu(z[n][j]) * z[n][hidden + j]."""
+GATE_ACTIVATIONS = {"silu": 0, "relu": 1, "gelu_tanh": 2}
+
+
+def gated_unit(z: torch.Tensor, act: torch.Tensor, n_rows: int, hidden: int, fast: bool = False,
+               activation: str = "silu") -> None:
+    """act[n][j] = f(z[n][j]) * z[n][hidden + j] with f = silu, relu or the tanh form of gelu."""
+    _need(activation in GATE_ACTIVATIONS, f"gated unit: activation {activation!r} is none of {sorted(GATE_ACTIVATIONS)}")
     _need_cuda(z, act)
     _need(z.dtype == act.dtype and z.dim() == 2 and act.dim() == 2 and z.stride(1) == 1 and act.stride(1) == 1
           and z.shape[1] >= 2 * hidden and act.shape[1] >= hidden and z.shape[0] >= n_rows and act.shape[0] >= n_rows,
           "z must be [>=n_rows, >=2 * hidden] and act [>=n_rows, >=hidden], one dtype")
     rc = library.kernels().mgpt_gated_unit(_ptr(z), z.stride(0), _ptr(act), act.stride(0), n_rows, hidden,
-                                           _dtype_code(z), int(fast), _stream())
+                                           _dtype_code(z), int(fast), GATE_ACTIVATIONS[activation], _stream())
     _check(rc, "gated_unit")
 
 
@@ -1217,3 +1224,175 @@ def grouped_linear_tiled(a: torch.Tensor, w: torch.Tensor, tile_expert: torch.Te
         return False
     _check(rc, "linear_mfma_grouped")
     return True
+
+
+# ---------------------------------------------------------------- root-mean-square norms, rotation, decaying state
+RMS_GATES = {None: 0, "silu": 1, "sigmoid": 2}
+
+
+def _rows_2d(name: str, t: torch.Tensor, n_rows: int) -> None:
+    _need(t.dim() == 2 and t.stride(1) == 1 and t.shape[0] >= n_rows and t.dtype in (torch.float32, torch.bfloat16),
+          f"{name} must be float32 or bfloat16 rows [>= {n_rows}, ...] with unit column stride")
+
+
+def rms_norm(x: torch.Tensor, gain: Optional[torch.Tensor], out: torch.Tensor, n_rows: int, eps: float, width: int,
+             offset: float = 0.0, mult: float = 1.0, rows: Optional[torch.Tensor] = None, groups: int = 1,
+             x_group_stride: Optional[int] = None, out_group_stride: Optional[int] = None,
+             gate: Optional[torch.Tensor] = None, gate_act: Optional[str] = None, accumulate: bool = False,
+             zero: Optional[torch.Tensor] = None) -> None:
+    """out[i, g] = (out[i, g] +) mult * x[r, g] / sqrt(mean(x[r, g]^2) + eps) * (offset + gain[g]) (* act(gate[i, g]))
+    with r = rows[i] or i; a row holds `groups` segments of `width` values, x_group_stride / out_group_stride
+    apart (default: width).  gain: float32 [groups * width] or None.  gate: laid out like out.  zero: float32 rows
+    that are cleared on the way (row i for every i)."""
+    _need_cuda(x, gain, out, rows, gate, zero)
+    xs = width if x_group_stride is None else int(x_group_stride)
+    os_ = width if out_group_stride is None else int(out_group_stride)
+    _rows_2d("rms_norm out", out, n_rows)
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.dtype in (torch.float32, torch.bfloat16), "rms_norm input must be rows")
+    _need(groups >= 1 and width >= 1 and xs >= width and os_ >= width, "rms_norm: segments overlap")
+    _need(x.shape[1] >= (groups - 1) * xs + width and out.shape[1] >= (groups - 1) * os_ + width,
+          "rms_norm: a row is shorter than its segments")
+    _need(gain is None or (gain.dtype == torch.float32 and gain.is_contiguous() and gain.numel() == groups * width),
+          "rms_norm gain must be float32 [groups * width]")
+    if rows is None:
+        _need(x.shape[0] >= n_rows, "rms_norm input has fewer rows than asked for")
+    else:
+        _need_i32("rows", rows, n_rows)
+    if gate is not None:
+        _rows_2d("rms_norm gate", gate, n_rows)
+        _need(gate.shape[1] >= (groups - 1) * os_ + width and gate_act in RMS_GATES, "rms_norm gate: too narrow, or unknown activation")
+    zero_width = 0
+    if zero is not None:
+        _need(zero.dtype == torch.float32 and zero.dim() == 2 and zero.stride(1) == 1 and zero.shape[0] >= n_rows,
+              "rms_norm: the buffer to clear must be float32 rows")
+        zero_width = zero.shape[1]
+    rc = library.kernels().mgpt_rms_norm(
+        _ptr(x), _dtype_code(x), x.stride(0), _ptr(rows), _ptr(gain), float(offset), float(eps), float(mult),
+        _ptr(gate), _dtype_code(gate) if gate is not None else 0, gate.stride(0) if gate is not None else 0,
+        RMS_GATES[gate_act if gate is not None else None], _ptr(out), _dtype_code(out), out.stride(0), int(accumulate),
+        _ptr(zero), zero.stride(0) if zero is not None else 0, zero_width, n_rows, groups, xs, os_, width, _stream())
+    _check(rc, "rms_norm")
+
+
+MAX_NORM_BRANCHES = 4
+
+
+def rms_post_norm(branches, x: torch.Tensor, gain_post: torch.Tensor, n_rows: int, eps: float, offset: float,
+                  mult: float, gain_next: Optional[torch.Tensor] = None, h: Optional[torch.Tensor] = None) -> None:
+    """branches: [(y float32 [rows, width], gain float32 [width] or None), ...].  With several branches
+    y = mean_b unit(y_b) * gain_b, else y = y_0; x += mult * unit(y) * (offset + gain_post); with gain_next
+    h = unit(x) * (offset + gain_next); every y_b is cleared.  unit(v) = v / sqrt(mean(v^2) + eps)."""
+    nb = len(branches)
+    _need(1 <= nb <= MAX_NORM_BRANCHES, f"rms_post_norm takes 1 to {MAX_NORM_BRANCHES} branches")
+    width = x.shape[1]
+    _need(x.dtype == torch.float32 and x.is_contiguous() and x.shape[0] >= n_rows, "rms_post_norm: x must be dense float32 rows")
+    ys, gs = [], []
+    for y, g in branches:
+        _need_cuda(y, g)
+        _need(y.dtype == torch.float32 and y.is_contiguous() and y.shape[1] == width and y.shape[0] >= n_rows,
+              "rms_post_norm: a branch must be dense float32 rows as wide as x")
+        _need(nb == 1 or (g is not None and g.dtype == torch.float32 and g.numel() == width and g.is_contiguous()),
+              "rms_post_norm: several branches need a float32 gain each")
+        ys.append(_ptr(y))
+        gs.append(_ptr(g) if nb > 1 else None)
+    ys += [None] * (MAX_NORM_BRANCHES - nb)
+    gs += [None] * (MAX_NORM_BRANCHES - nb)
+    for g in (gain_post, gain_next):
+        _need(g is None or (g.dtype == torch.float32 and g.numel() == width and g.is_contiguous()), "rms_post_norm: gains are float32 [width]")
+    _need(gain_post is not None, "rms_post_norm needs the gain of the norm behind the sublayer")
+    if gain_next is not None:
+        _need(h is not None and h.is_contiguous() and h.shape[1] == width and h.shape[0] >= n_rows
+              and h.dtype in (torch.float32, torch.bfloat16), "rms_post_norm: h must be dense rows as wide as x")
+    _need_cuda(x, gain_post, gain_next, h)
+    rc = library.kernels().mgpt_rms_post_norm(
+        *ys, *gs, nb, 1.0 / nb, _ptr(x), _ptr(gain_post), float(offset), float(eps), float(mult), _ptr(gain_next),
+        _ptr(h) if gain_next is not None else None, _dtype_code(h) if gain_next is not None else 0, n_rows, width, _stream())
+    _check(rc, "rms_post_norm")
+
+
+def qk_prepare(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int, n_kv_head: int, head_dim: int,
+               value_dim: int, head_stride: int, n_tokens: int, positions: Optional[torch.Tensor] = None,
+               freq: Optional[torch.Tensor] = None, norm_eps: Optional[float] = None,
+               mix_lambda: Optional[torch.Tensor] = None, v_other: Optional[torch.Tensor] = None, mix_mode: int = 0,
+               k_pool: Optional[torch.Tensor] = None, v_pool: Optional[torch.Tensor] = None,
+               slot_mapping: Optional[torch.Tensor] = None) -> None:
+    """Projected queries, keys and values of a step's tokens (rows of z; q heads at q_off, k heads at k_off, v heads
+    at v_off, head_stride channels apart) made ready for attention: q and k rotated by position with the float32
+    frequencies `freq` [rot_dims / 2] (pairs (i, i + rot_dims / 2)), then divided by their root mean square over
+    head_dim channels if norm_eps is given; v kept for other layers in v_other (heads value_dim apart; mix_mode 1) or mixed with what
+    lies there, (1 - lambda) v + lambda v_other (mix_mode 2); q back in place, k and v into their pages."""
+    _need_cuda(z, positions, freq, mix_lambda, v_other, k_pool, v_pool, slot_mapping)
+    _rows_2d("qk_prepare z", z, n_tokens)
+    rot_dims = 0
+    if freq is not None:
+        _need(freq.dtype == torch.float32 and freq.is_contiguous() and positions is not None, "rotation needs float32 frequencies and positions")
+        _need_i32("positions", positions, n_tokens)
+        rot_dims = 2 * freq.numel()
+    kv_span = (n_kv_head - 1) * head_stride
+    _need(z.shape[1] >= max(q_off + (n_head - 1) * head_stride + head_dim, k_off + kv_span + head_dim,
+                            v_off + kv_span + head_stride if k_pool is not None else 0), "qk_prepare: z is too narrow")
+    page_size = 0
+    if k_pool is not None:
+        _need(v_pool is not None and k_pool.dtype == z.dtype and v_pool.dtype == z.dtype and k_pool.dim() == 4
+              and k_pool.shape[1] == n_kv_head and k_pool.shape[3] == head_stride and k_pool.is_contiguous()
+              and v_pool.shape == k_pool.shape and v_pool.is_contiguous(),
+              "qk_prepare: pools must be [pages, kv heads, page, head stride] in z's dtype")
+        _need_i32("slot_mapping", slot_mapping, n_tokens)
+        page_size = k_pool.shape[2]
+    if mix_mode:
+        _need(v_other is not None and v_other.dtype == z.dtype and v_other.dim() == 2 and v_other.stride(1) == 1
+              and v_other.shape[0] >= n_tokens and v_other.shape[1] >= n_kv_head * value_dim,
+              "qk_prepare: the shared values must be rows of all kv heads in z's dtype")
+        _need(mix_mode == 1 or (mix_lambda is not None and mix_lambda.dtype == torch.float32 and mix_lambda.numel() >= 1),
+              "qk_prepare: mixing needs a float32 lambda")
+    rc = library.kernels().mgpt_qk_prepare(
+        _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, n_head, n_kv_head, head_dim, value_dim, head_stride,
+        _ptr(positions), _ptr(freq), rot_dims, -1.0 if norm_eps is None else float(norm_eps), _ptr(mix_lambda),
+        _ptr(v_other), v_other.stride(0) if v_other is not None else 0, int(mix_mode), _ptr(k_pool), _ptr(v_pool),
+        _ptr(slot_mapping), page_size, n_tokens, _stream())
+    _check(rc, "qk_prepare")
+
+
+def head_gate(y: torch.Tensor, gate: torch.Tensor, n_rows: int, n_head: int, width: int, head_stride: int) -> None:
+    """y[n, h * head_stride + c] *= sigmoid(gate[n, h]) for c < width."""
+    _need_cuda(y, gate)
+    _rows_2d("head_gate y", y, n_rows)
+    _rows_2d("head_gate gate", gate, n_rows)
+    _need(y.shape[1] >= (n_head - 1) * head_stride + width and gate.shape[1] >= n_head, "head_gate: rows too narrow")
+    rc = library.kernels().mgpt_head_gate(_ptr(y), _dtype_code(y), y.stride(0), head_stride, width, _ptr(gate),
+                                          _dtype_code(gate), gate.stride(0), n_rows, n_head, _stream())
+    _check(rc, "head_gate")
+
+
+def decay_state(z: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, n_head: int, head_dim: int,
+                value_dim: int, decay: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+                n_req: int, positions: torch.Tensor, out: torch.Tensor, silu_inputs: bool = False,
+                freq: Optional[torch.Tensor] = None, k_scale: float = 1.0, norm_eps: Optional[float] = None) -> None:
+    """Per request and head the state S [head_dim, value_dim] (float32, in the request's slot of `state`, zero
+    before position 0) goes over the request's tokens of this step: S = decay_h S + k v^T, o = S^T q.  q, k, v
+    (and a gate at g_off, -1 for none) are columns of z's rows; silu_inputs passes them through silu first; freq
+    rotates q and k by position; k is multiplied by k_scale.  out[n, h] = o (divided by its root mean square with
+    norm_eps given, times silu(gate) with a gate), float32 or z's dtype."""
+    _need_cuda(z, decay, state, state_slots, cu_q, positions, out, freq)
+    n_tokens = 0
+    _rows_2d("decay_state z", z, n_tokens)
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_head * value_dim
+          and out.dtype in (torch.float32, torch.bfloat16), "decay_state: out must be rows of all heads' values")
+    _need(z.shape[1] >= max(q_off, k_off) + n_head * head_dim and z.shape[1] >= max(v_off, g_off) + n_head * value_dim,
+          "decay_state: z is too narrow")
+    _need(decay.dtype == torch.float32 and decay.numel() == n_head, "decay_state: one float32 decay per head")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+          and state.shape[1] == n_head * head_dim * value_dim, "decay_state: state must be [slots, heads * dim * vdim] float32")
+    _need_i32("state_slots", state_slots, n_req)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need(positions.dtype == torch.int32 and positions.is_contiguous(), "positions must be int32")
+    _need(0 < head_dim <= 256 and 0 < value_dim <= 256, "decay_state takes head sizes up to 256")
+    rot_dims = 0
+    if freq is not None:
+        _need(freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= head_dim, "decay_state: bad frequencies")
+        rot_dims = 2 * freq.numel()
+    rc = library.kernels().mgpt_decay_state(
+        _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, g_off, n_head, head_dim, value_dim, int(silu_inputs),
+        _ptr(positions), _ptr(freq), rot_dims, float(k_scale), _ptr(decay), _ptr(state), _ptr(state_slots), _ptr(cu_q),
+        n_req, -1.0 if norm_eps is None else float(norm_eps), _ptr(out), _dtype_code(out), out.stride(0), _stream())
+    _check(rc, "decay_state")

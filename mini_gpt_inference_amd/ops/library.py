@@ -39,7 +39,7 @@ def kernels() -> ctypes.CDLL:
         lib.mgpt_layernorm.argtypes = [P, P, P, P, P, I, I, F, I, P]
         lib.mgpt_linear_generic.argtypes = [P, I, L, P, I, P, P, I, L, I, I, I, I, P]
         lib.mgpt_kv_write.argtypes = [P, I, L, I, I, P, P, P, I, I, I, I, P]
-        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, P]
+        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, F, P]
         lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P, P, I, P]
         lib.mgpt_sample_advance.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P,
                                             P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P, P, I, P]
@@ -158,7 +158,13 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_heads_linear": [P, L, P, P, L, P, L, I, I, I, I, I, I, P],
         "mgpt_heads_linear_mfma": [P, L, P, P, L, P, L, I, I, I, I, P],
         # gated feed-forwards and experts
-        "mgpt_gated_unit": [P, L, P, L, I, I, I, I, P],
+        "mgpt_gated_unit": [P, L, P, L, I, I, I, I, I, P],
+        # root-mean-square norms, rotation and the rest in front of attention, decaying state
+        "mgpt_rms_norm": [P, I, L, P, P, F, F, F, P, I, L, I, P, I, L, I, P, L, I, I, I, I, I, I, P],
+        "mgpt_rms_post_norm": [P, P, P, P, P, P, P, P, I, F, P, P, F, F, F, P, P, I, I, I, P],
+        "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, P],
+        "mgpt_head_gate": [P, I, L, I, I, P, I, L, I, I, P],
+        "mgpt_decay_state": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, F, P, I, L, P],
         "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, P, I, I, I, P],
         "mgpt_gather_rows": [P, L, P, P, L, I, I, P],
         "mgpt_linear_mfma_grouped": [P, L, P, L, P, P, I, P, I, L, I, I, I, P],

@@ -143,3 +143,71 @@ class HyperConnections(Arrangement):
         if self.has_feed_forward:
             feed_forward = parts["feed_forward"]
             self._sublayer(ctx, x, "2", parts["norm2"], lambda h, y: feed_forward.forward_add(ctx, h, y))
+
+
+@register_arrangement("sandwich_norm")
+class SandwichNorm(Arrangement):
+    """A layer whose sublayers are normed on both sides and whose additions to the residual are scaled:
+
+        x <- x + m * norm1b(mixer(norm1(x)));   x <- x + m * norm2b(ff(norm2(x)))
+
+    with m = `residual_mult`; the feed-forward half is optional.  With `branches` = B > 1 the mixer is
+    B mixers side by side that read the same norm1(x) (roles mixer0 .. mixer{B-1}), and what norm1b
+    sees is the mean of their outputs, each first normed with a gain of its own (roles join0 ..):
+    (1 / B) * sum_b join_b(mixer_b(h)).  All norms are RMS norms (kind "rms_norm"); the norms around
+    the sublayers share one eps and one way of storing the gain, the joins have plain gains.
+
+    The sublayers are the framework's ordinary parts: they add their output into a cleared float32
+    buffer.  One kernel stands between two sublayers: it joins the branches, norms the sum, adds it
+    to the residual, computes the next sublayer's input norm and clears the buffers again."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, residual_mult: float = 1.0, feed_forward: bool = True, branches: int = 1) -> None:
+        self.width, self.mult = int(width), float(residual_mult)
+        self.has_feed_forward, self.branches = bool(feed_forward), int(branches)
+        if not 1 <= self.branches <= kernels.MAX_NORM_BRANCHES:
+            raise ValueError(f"{self.branches} parallel mixers: the kernels take 1 to {kernels.MAX_NORM_BRANCHES}")
+        if self.branches == 1:
+            self.mixer_roles, self.join_roles = ("mixer",), ()
+        else:
+            self.mixer_roles = tuple(f"mixer{b}" for b in range(self.branches))
+            self.join_roles = tuple(f"join{b}" for b in range(self.branches))
+        self.roles = ("norm1",) + self.mixer_roles + self.join_roles + ("norm1b",)
+        if self.has_feed_forward:
+            self.roles += ("norm2", "feed_forward", "norm2b")
+        self._checked = False
+
+    def _check(self, parts) -> None:
+        around = [parts[r] for r in self.roles if r.startswith("norm")]
+        for p in around + [parts[r] for r in self.join_roles]:
+            if not (hasattr(p, "offset") and getattr(p, "has_weight", False) and p.width == self.width):
+                raise ValueError("a sandwich-norm layer takes RMS norms with gains as wide as the model")
+        if len({(p.eps, p.offset) for p in around}) != 1 or any(parts[r].eps != around[0].eps for r in self.join_roles):
+            raise ValueError("the norms of a sandwich-norm layer share one eps and one way of storing the gain")
+        if any(parts[r].offset != 0.0 for r in self.join_roles):
+            raise ValueError("the norms that join parallel mixers have plain gains")
+        self._checked = True
+
+    def run(self, ctx, x, parts, bindings, position) -> None:
+        if not self._checked:
+            self._check(parts)
+        n, ws, B = ctx.n_rows, ctx.workspace, self.branches
+        norm1 = parts["norm1"]
+        flat = ws.get("sublayer_sums", B * n, self.width, torch.float32)[:B * n]
+        ys = flat.view(B, n, self.width)
+        h = ws.get("normed", n, self.width, ctx.dtype)
+        norm1.forward(ctx, x, h, n, zero=flat.view(n, B * self.width))
+        for b, role in enumerate(self.mixer_roles):
+            parts[role].forward_add(ctx, h, ys[b], bindings[role], position)
+        joins = [(ys[b], parts[self.join_roles[b]].weight if B > 1 else None) for b in range(B)]
+        norm1b = parts["norm1b"]
+        if not self.has_feed_forward:
+            kernels.rms_post_norm(joins, x, norm1b.weight, n, norm1b.eps, norm1b.offset, self.mult)
+            return
+        kernels.rms_post_norm(joins, x, norm1b.weight, n, norm1b.eps, norm1b.offset, self.mult,
+                              gain_next=parts["norm2"].weight, h=h)
+        parts["feed_forward"].forward_add(ctx, h, ys[0])
+        norm2b = parts["norm2b"]
+        kernels.rms_post_norm([(ys[0], None)], x, norm2b.weight, n, norm2b.eps, norm2b.offset, self.mult)

@@ -85,12 +85,12 @@ class DenseMLP(FeedForward):
 
 
 def _gated(ctx: StepContext, h, in_weight: torch.Tensor, down_weight: torch.Tensor, x: torch.Tensor, n: int,
-           hidden: int) -> None:
-    """x += (silu(h Wgate^T) * (h Wup^T)) Wdown^T with the gate and up matrices stacked in in_weight."""
+           hidden: int, activation: str = "silu") -> None:
+    """x += (act(h Wgate^T) * (h Wup^T)) Wdown^T with the gate and up matrices stacked in in_weight."""
     z = ctx.workspace.get("gated_z", n, 2 * hidden, ctx.dtype)
     linear(ctx, h, in_weight, None, z, n)
     act = ctx.workspace.get("gated_act", n, hidden, ctx.dtype)
-    kernels.gated_unit(z, act, n, hidden, fast=not ctx.exact)
+    kernels.gated_unit(z, act, n, hidden, fast=not ctx.exact, activation=activation)
     linear_add(ctx, act, down_weight, None, x, n)
 
 
@@ -106,14 +106,17 @@ def _stack_gate_up(part: Part, tensors, gate: str, up: str):
 
 @register_feed_forward("gated_mlp")
 class GatedMLP(FeedForward):
-    """m = (silu(h Wgate^T) * (h Wup^T)) Wdown^T, silu(v) = v sigmoid(v), no biases; the unit's
-    nonlinearity and product in float32."""
+    """m = (act(h Wgate^T) * (h Wup^T)) Wdown^T, no biases; act is silu(v) = v sigmoid(v) unless
+    `activation` names relu or gelu_tanh; the unit's nonlinearity and product in float32."""
 
     graph_safe = True
     plan_safe = True
 
-    def __init__(self, width: int, hidden: int) -> None:
+    def __init__(self, width: int, hidden: int, activation: str = "silu") -> None:
         self.width, self.hidden = int(width), int(hidden)
+        if activation not in kernels.GATE_ACTIVATIONS:
+            raise ValueError(f"gated unit: activation {activation!r} is none of {sorted(kernels.GATE_ACTIVATIONS)}")
+        self.activation = activation
         self.in_weight = None
 
     def weight_requests(self) -> Dict[str, WeightRequest]:
@@ -128,7 +131,7 @@ class GatedMLP(FeedForward):
 
     def forward_add(self, ctx: StepContext, h, x: torch.Tensor) -> None:
         plain_residual(ctx, h, x)
-        _gated(ctx, h, self.in_weight, self.down_weight, x, ctx.n_rows, self.hidden)
+        _gated(ctx, h, self.in_weight, self.down_weight, x, ctx.n_rows, self.hidden, self.activation)
 
 
 @register_feed_forward("table_experts")

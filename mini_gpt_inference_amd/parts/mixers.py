@@ -9,8 +9,8 @@ import torch
 from ..ops import attention as attention_ops
 from ..ops import kernels, residual
 from ..ops.linear import LazyNorm, as_tensor, linear, linear_add, packed_weight, plain_residual
-from .base import (CacheBinding, KVNeed, MATRIX, Part, StateNeed, StepContext, VECTOR, WeightRequest,
-                   register_mixer)
+from .base import (CacheBinding, KVNeed, MATRIX, POSITIONS, Part, PartSpec, StateNeed, StepContext, VECTOR,
+                   WeightRequest, register_mixer)
 from .positions import PositionEncoding
 
 
@@ -237,4 +237,236 @@ class LatentAttention(Mixer):
                                       sinks=self.sink)
         y = ws.get("attn_out", n, self.g_width, ctx.dtype)
         kernels.heads_linear(o_lat, self.uv_heads, y, n, gate=z[:, self.q_width:self.q_width + self.g_width], fast=fast)
+        linear_add(ctx, y, self.out_weight, None, x, n)
+
+
+def _own_rotation(rotary: Optional[dict]) -> Optional[PositionEncoding]:
+    """A mixer's own position encoding from its parameters ({"kind": ..., constants}), through the
+    registry of position encodings; None: the mixer does not rotate."""
+    if not rotary:
+        return None
+    params = dict(rotary)
+    part = POSITIONS.build(PartSpec(params.pop("kind", "rotary_half"), params))
+    if not hasattr(part, "frequencies"):
+        raise ValueError("a mixer's own rotation must give a frequency table (frequencies(device))")
+    return part
+
+
+@register_mixer("gated_attention")
+class GatedAttention(Mixer):
+    """Causal softmax attention over the paged cache with grouped key/value heads, a query/key size
+    D that may differ from the value size E, and these optional steps, each a parameter:
+
+    q = h Wq^T (+ b), k = h Wk^T (+ b), v = h Wv^T (+ b);  q, k rotated by position (`rotary`: the
+    mixer's own rotation);  q, k divided by their root mean square per head (`qk_norm_eps`);
+    v <- (1 - lambda) v + lambda v_other with v_other the values that the layer with
+    value_mix="keep" made for the same token (value_mix="mix"; lambda is the tensor `mix`); what is
+    cached is the rotated, normed key and the mixed value.  S = (q . k) * scale, capped as
+    cap * tanh(S / cap) (`softcap`), softmax in float32 over the keys at positions <= the query's;
+    head a's output times sigmoid(h Wg^T)_a, one number per head (`head_gate`); out = y Wo^T, added
+    into the residual.
+
+    The cache keeps keys and values in pages of one head size, so both are laid out with
+    max(D, E) channels a head (rounded up to what the bfloat16 attention kernels take), the
+    channels beyond a head's own being zeros that the stacked projection matrix makes by itself."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, n_head: int, n_kv_head: int, head_dim: int, value_dim: int, scale: float,
+                 bias: bool = False, rotary: Optional[dict] = None, qk_norm_eps: Optional[float] = None,
+                 softcap: float = 0.0, head_gate: bool = False, value_mix: Optional[str] = None,
+                 share: str = "values") -> None:
+        self.width, self.n_head, self.n_kv_head = int(width), int(n_head), int(n_kv_head)
+        self.head_dim, self.value_dim, self.scale = int(head_dim), int(value_dim), float(scale)
+        self.has_bias, self.has_gate = bool(bias), bool(head_gate)
+        self.rotation = _own_rotation(rotary)
+        self.qk_norm_eps = None if qk_norm_eps is None else float(qk_norm_eps)
+        self.softcap = float(softcap or 0.0)
+        if value_mix not in (None, "keep", "mix"):
+            raise ValueError(f"value_mix {value_mix!r} is none of None, 'keep', 'mix'")
+        self.value_mix, self.share = value_mix, str(share)
+        if self.n_head % self.n_kv_head != 0:
+            raise ValueError("n_head must be a multiple of n_kv_head")
+        if self.rotation is not None and self.rotation.dims > self.head_dim:
+            raise ValueError(f"rotation over {self.rotation.dims} channels of heads of {self.head_dim}")
+        size = max(self.head_dim, self.value_dim)
+        self.head_stride = -(-size // 32) * 32 if size <= 128 else -(-size // 8) * 8
+        if self.head_stride > 512:
+            raise ValueError(f"head size {size}: the attention kernels take up to 512")
+        s = self.head_stride
+        self.q_off, self.k_off = 0, self.n_head * s
+        self.v_off = self.k_off + self.n_kv_head * s
+        self.g_off = self.v_off + self.n_kv_head * s
+        self.in_rows = -(-(self.g_off + (self.n_head if self.has_gate else 0)) // 16) * 16
+        self.in_weight = self.in_bias = self.out_padded = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        H, G, D, E, W = self.n_head, self.n_kv_head, self.head_dim, self.value_dim, self.width
+        req = {"q_weight": WeightRequest((H * D, W), MATRIX), "k_weight": WeightRequest((G * D, W), MATRIX),
+               "v_weight": WeightRequest((G * E, W), MATRIX), "out_weight": WeightRequest((W, H * E), MATRIX)}
+        if self.has_bias:
+            req.update(q_bias=WeightRequest((H * D,), VECTOR), k_bias=WeightRequest((G * D,), VECTOR),
+                       v_bias=WeightRequest((G * E,), VECTOR))
+        if self.has_gate:
+            req["gate_weight"] = WeightRequest((H, W), MATRIX)
+        if self.value_mix is not None:
+            req["mix"] = WeightRequest((), VECTOR)
+        return req
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        H, G, D, E, W, s = self.n_head, self.n_kv_head, self.head_dim, self.value_dim, self.width, self.head_stride
+        q = tensors["q_weight"]
+        joint = torch.zeros((self.in_rows, W), dtype=q.dtype, device=q.device)
+        views = {}
+
+        def place(name: str, at: int, heads: int, size: int) -> None:
+            block = joint[at:at + heads * s].view(heads, s, W)[:, :size]
+            block.copy_(tensors[name].view(heads, size, W))
+            views[name] = block
+
+        place("q_weight", self.q_off, H, D)
+        place("k_weight", self.k_off, G, D)
+        place("v_weight", self.v_off, G, E)
+        if self.has_gate:
+            joint[self.g_off:self.g_off + H].copy_(tensors["gate_weight"])
+            views["gate_weight"] = joint[self.g_off:self.g_off + H]
+        self.in_weight = joint
+        if self.has_bias:
+            bias = torch.zeros(self.in_rows, dtype=torch.float32, device=q.device)
+            for name, at, heads, size in (("q_bias", self.q_off, H, D), ("k_bias", self.k_off, G, D),
+                                          ("v_bias", self.v_off, G, E)):
+                bias[at:at + heads * s].view(heads, s)[:, :size].copy_(tensors[name].view(heads, size))
+            self.in_bias = bias
+        out = tensors["out_weight"]
+        padded = torch.zeros((W, H * s), dtype=out.dtype, device=out.device)
+        padded.view(W, H, s)[:, :, :E].copy_(out.view(W, H, E))
+        self.out_padded = padded
+        views["out_weight"] = padded.view(W, H, s)[:, :, :E]
+        for name, view in views.items():
+            setattr(self, name, view)
+        return views
+
+    def cache_need(self) -> KVNeed:
+        return KVNeed(self.n_kv_head, self.head_stride, 0)
+
+    def token_matrix_elements(self) -> int:
+        return self.in_weight.numel() + self.out_padded.numel() if self.in_weight is not None else 0
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        if not binding.writes:
+            raise ValueError("gated attention keeps its own keys and values")
+        plain_residual(ctx, h, x)
+        n, ws, s = ctx.n_rows, ctx.workspace, self.head_stride
+        z = ws.get("gated_attention_in", n, self.in_rows, ctx.dtype)
+        linear(ctx, h, self.in_weight, self.in_bias, z, n)
+        group = ctx.groups[binding.group]
+        k_pool, v_pool = group.k_pools[binding.index], group.v_pools[binding.index]
+        other, mode = None, 0
+        if self.value_mix is not None:
+            other = ws.get("shared_" + self.share, n, self.n_kv_head * self.value_dim, ctx.dtype)
+            mode = 1 if self.value_mix == "keep" else 2
+        kernels.qk_prepare(z, self.q_off, self.k_off, self.v_off, self.n_head, self.n_kv_head, self.head_dim, self.value_dim, s, n,
+                           positions=ctx.positions,
+                           freq=self.rotation.frequencies(z.device) if self.rotation is not None else None,
+                           norm_eps=self.qk_norm_eps, mix_lambda=self.mix if mode == 2 else None, v_other=other,
+                           mix_mode=mode, k_pool=k_pool, v_pool=v_pool, slot_mapping=group.slot_mapping)
+        y = ws.get("attn_out", n, self.n_head * s, ctx.dtype)
+        attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, 0, softcap=self.softcap)
+        if self.has_gate:
+            kernels.head_gate(y, z[:, self.g_off:], n, self.n_head, s, s)
+        linear_add(ctx, y, self.out_padded, None, x, n)
+
+
+@register_mixer("decay_state")
+class DecayStateMixer(Mixer):
+    """Linear attention with a fixed decay per head: no softmax, no denominator, and instead of a
+    cache one float32 matrix per request and head.
+
+    q = f(h Wq^T), k = f(h Wk^T) [H, D], v = f(h Wv^T) [H, E] with f the identity or silu
+    (`input_activation`); q and k rotated by position (`rotary`); k times `k_scale`;
+    S_t = decay_a S_(t-1) + k_t v_t^T, o_t = S_t^T q_t per head a, S zero before the first token.
+    Then either each head's o divided by its root mean square (`head_norm_eps`) and the heads
+    multiplied by silu(h Wg^T), or (`out_norm_eps`) the concatenated heads RMS-normed with the
+    weight `norm_weight` and multiplied by sigmoid(h Wg^T); out = y Wo^T, added into the residual.
+    From the rotation on everything is float32 up to y."""
+
+    graph_safe = True
+    plan_safe = True
+
+    def __init__(self, width: int, n_head: int, head_dim: int, value_dim: int, decay, rotary: Optional[dict] = None,
+                 k_scale: float = 1.0, input_activation: Optional[str] = None, head_norm_eps: Optional[float] = None,
+                 out_norm_eps: Optional[float] = None) -> None:
+        self.width, self.n_head, self.head_dim, self.value_dim = int(width), int(n_head), int(head_dim), int(value_dim)
+        self.decay_values = [float(d) for d in decay]
+        if len(self.decay_values) != self.n_head:
+            raise ValueError(f"{len(self.decay_values)} decays for {self.n_head} heads")
+        if input_activation not in (None, "silu"):
+            raise ValueError(f"input activation {input_activation!r} is neither None nor 'silu'")
+        if (head_norm_eps is None) == (out_norm_eps is None):
+            raise ValueError("exactly one of head_norm_eps and out_norm_eps says how the heads' outputs are normed")
+        if not (0 < self.head_dim <= 256 and 0 < self.value_dim <= 256):
+            raise ValueError("the state kernel takes head sizes up to 256")
+        self.rotation = _own_rotation(rotary)
+        if self.rotation is not None and self.rotation.dims > self.head_dim:
+            raise ValueError(f"rotation over {self.rotation.dims} channels of heads of {self.head_dim}")
+        self.k_scale, self.silu_inputs = float(k_scale), input_activation == "silu"
+        self.head_norm_eps = None if head_norm_eps is None else float(head_norm_eps)
+        self.out_norm_eps = None if out_norm_eps is None else float(out_norm_eps)
+        self.qk_width, self.v_width = self.n_head * self.head_dim, self.n_head * self.value_dim
+        self.k_off, self.v_off, self.g_off = self.qk_width, 2 * self.qk_width, 2 * self.qk_width + self.v_width
+        self.in_weight = None
+        self._decay: Dict[torch.device, torch.Tensor] = {}
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        W = self.width
+        req = {"q_weight": WeightRequest((self.qk_width, W), MATRIX), "k_weight": WeightRequest((self.qk_width, W), MATRIX),
+               "v_weight": WeightRequest((self.v_width, W), MATRIX), "gate_weight": WeightRequest((self.v_width, W), MATRIX),
+               "out_weight": WeightRequest((W, self.v_width), MATRIX)}
+        if self.out_norm_eps is not None:
+            req["norm_weight"] = WeightRequest((self.v_width,), VECTOR)
+        return req
+
+    def bind(self, tensors):
+        super().bind(tensors)
+        names = ["q_weight", "k_weight", "v_weight", "gate_weight"]
+        self.in_weight = torch.cat([tensors[n] for n in names], dim=0).contiguous()
+        views, at = {}, 0
+        for n in names:
+            rows = tensors[n].shape[0]
+            views[n] = self.in_weight[at:at + rows]
+            setattr(self, n, views[n])
+            at += rows
+        return views
+
+    def cache_need(self) -> StateNeed:
+        return StateNeed(self.n_head * self.head_dim * self.value_dim)
+
+    def _decays(self, device: torch.device) -> torch.Tensor:
+        d = self._decay.get(device)
+        if d is None:
+            d = self._decay[device] = torch.tensor(self.decay_values, dtype=torch.float32, device=device)
+        return d
+
+    def forward_add(self, ctx: StepContext, h, x: torch.Tensor, binding: CacheBinding,
+                    position: PositionEncoding) -> None:
+        if binding.kind != "state":
+            raise ValueError("a decaying-state mixer needs a state pool")
+        plain_residual(ctx, h, x)
+        n, ws = ctx.n_rows, ctx.workspace
+        z = ws.get("decay_state_in", n, self.in_weight.shape[0], ctx.dtype)
+        linear(ctx, h, self.in_weight, None, z, n)
+        y = ws.get("decay_state_out", n, self.v_width, ctx.dtype)
+        gated_here = self.head_norm_eps is not None
+        o = y if gated_here else ws.get("decay_state_sums", n, self.v_width, torch.float32)
+        kernels.decay_state(z, 0, self.k_off, self.v_off, self.g_off if gated_here else -1, self.n_head, self.head_dim,
+                            self.value_dim, self._decays(z.device), ctx.state_pools[binding.index], ctx.state_slots,
+                            ctx.cu_q, ctx.cu_q.numel() - 1, ctx.positions, o, silu_inputs=self.silu_inputs,
+                            freq=self.rotation.frequencies(z.device) if self.rotation is not None else None,
+                            k_scale=self.k_scale, norm_eps=self.head_norm_eps)
+        if not gated_here:
+            kernels.rms_norm(o, self.norm_weight, y, n, self.out_norm_eps, self.v_width, gate=z[:, self.g_off:],
+                             gate_act="sigmoid")
         linear_add(ctx, y, self.out_weight, None, x, n)

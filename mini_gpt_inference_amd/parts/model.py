@@ -84,6 +84,8 @@ class ModelSpec:
     streams: int = 1
     # (duplicate name, tensor it must equal): names a checkpoint may carry beside the tensor they alias
     tied_aliases: Tuple[Tuple[str, str], ...] = ()
+    # a norm applied to the embedded tokens before the first layer (in place, float32); None: none
+    embedding_norm: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)
@@ -181,6 +183,9 @@ class DecoderModel:
             self.layers.append(_Layer(arrangement, {role: _LAYER_REGISTRIES[category].build(part_spec)
                                                     for role, (category, part_spec) in ls.parts.items()}))
         self.final_norm = NORMS.build(spec.final_norm)
+        self.embedding_norm = NORMS.build(spec.embedding_norm) if spec.embedding_norm is not None else None
+        if self.embedding_norm is not None and spec.streams != 1:
+            raise ValueError("a norm behind the embedding goes with one residual stream")
         self.head = HEADS.build(spec.head)
         for i, run in enumerate(spec.order):
             if not (0 <= run.layer < len(self.layers)):
@@ -193,6 +198,8 @@ class DecoderModel:
     # ------------------------------------------------------------------ weights
     def _named_parts(self) -> List[Tuple[Part, PartSpec]]:
         pairs = [(self.embedding, self.spec.embedding), (self.position, self.spec.position)]
+        if self.embedding_norm is not None:
+            pairs.append((self.embedding_norm, self.spec.embedding_norm))
         for layer, ls in zip(self.layers, self.spec.layers):
             pairs += [(layer.parts[role], part_spec) for role, (_, part_spec) in ls.parts.items()]
             pairs.append((layer.arrangement, ls.arrangement))      # an arrangement may have tensors of its own
@@ -335,7 +342,7 @@ class DecoderModel:
     @property
     def graph_safe(self) -> bool:
         """Whether every part of the model allows a step to be captured in a HIP graph (Part.graph_safe)."""
-        parts = [self.embedding, self.position, self.final_norm, self.head]
+        parts = [self.embedding, self.position, self.embedding_norm, self.final_norm, self.head]
         for layer in self.layers:
             parts += [layer.arrangement, *layer.parts.values()]
         return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
@@ -343,7 +350,7 @@ class DecoderModel:
     @property
     def plan_safe(self) -> bool:
         """Whether every part of the model computes through the kernel library only (Part.plan_safe)."""
-        parts = [self.embedding, self.position, self.final_norm, self.head]
+        parts = [self.embedding, self.position, self.embedding_norm, self.final_norm, self.head]
         for layer in self.layers:
             parts += [layer.arrangement, *layer.parts.values()]
         return self.graph_safe and all(getattr(p, "plan_safe", False) for p in parts if p is not None)
@@ -360,6 +367,9 @@ class DecoderModel:
         ctx.pending = None
         ctx.pending_streams = None
         self.embedding.forward(ctx, self.position, x)
+        if self.embedding_norm is not None:
+            residual.settle(ctx, x, n)
+            self.embedding_norm.forward(ctx, x, x, n)
         for run, bindings in zip(self.spec.order, self.cache_layout.run_bindings):
             layer = self.layers[run.layer]
             if not getattr(layer.arrangement, "takes_pending_streams", False):

@@ -38,3 +38,30 @@ class LayerNorm(Part):
                 rows: Optional[torch.Tensor] = None) -> None:
         """out[i] = norm(x[rows[i]]) (or x[i]); x is the float32 residual stream."""
         kernels.layer_norm(x, self.weight, self.bias, out, n_rows, self.eps, rows)
+
+
+@register_norm("rms_norm")
+class RMSNorm(Part):
+    """y = x / sqrt(mean(x^2) + eps) * g over the last dim, statistics in float32.  g is the stored
+    weight, or one plus it for a weight stored as its distance from one (one_plus), or absent."""
+
+    graph_safe = True
+    plan_safe = True
+
+    category = "norm"
+
+    def __init__(self, width: int, eps: float, one_plus: bool = False, weight: bool = True) -> None:
+        self.width, self.eps = int(width), float(eps)
+        self.offset = 1.0 if one_plus else 0.0
+        self.has_weight = bool(weight)
+        self.weight: Optional[torch.Tensor] = None
+
+    def weight_requests(self) -> Dict[str, WeightRequest]:
+        return {"weight": WeightRequest((self.width,), VECTOR)} if self.has_weight else {}
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, out: torch.Tensor, n_rows: int,
+                rows: Optional[torch.Tensor] = None, zero: Optional[torch.Tensor] = None) -> None:
+        """out[i] = norm(x[rows[i]]) (or x[i]); out may be x itself (float32) or rows in the compute
+        dtype; `zero`: float32 rows that the same pass clears."""
+        kernels.rms_norm(x, self.weight, out, n_rows, self.eps, self.width, offset=self.offset if self.has_weight else 0.0,
+                         rows=rows, zero=zero)

@@ -58,3 +58,31 @@ class NoPositions(PositionEncoding):
 
     def __init__(self) -> None:
         pass
+
+
+@register_position("rotary_half")
+class RotaryHalf(PositionEncoding):
+    """Rotation of queries and keys by position, on the first `dims` channels of every head:
+    channel i is paired with channel i + dims/2, and at position p the pair (u, w) becomes
+    (u cos a - w sin a, w cos a + u sin a) with a = p * base^(-2i/dims) / factor (factor: linear
+    scaling of the positions).  The other channels pass unchanged.  A mixer that rotates owns one of
+    these (its constants are the mixer's); the kernels that apply it take the frequency table."""
+
+    graph_safe = True
+    plan_safe = True
+    rotates = True
+
+    def __init__(self, dims: int, base: float, factor: float = 1.0) -> None:
+        self.dims, self.base, self.factor = int(dims), float(base), float(factor)
+        if self.dims <= 0 or self.dims % 2 or self.base <= 0.0 or self.factor <= 0.0:
+            raise ValueError(f"rotation over {dims} channels with base {base} and factor {factor}")
+        self._freq: Dict[torch.device, torch.Tensor] = {}
+
+    def frequencies(self, device: torch.device) -> torch.Tensor:
+        """float32 [dims / 2]: the angle per position of every pair, computed in double precision."""
+        f = self._freq.get(device)
+        if f is None:
+            f = torch.tensor([self.base ** (-2.0 * i / self.dims) / self.factor for i in range(self.dims // 2)],
+                             dtype=torch.float64).to(torch.float32).to(device)
+            self._freq[device] = f
+        return f
