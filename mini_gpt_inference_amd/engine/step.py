@@ -360,8 +360,14 @@ class ModelRunner:
                     entry.plan.run()
                 self.num_planned_steps += 1
                 return entry.plan_logits
+            moved = self.workspace.moved
             with library.record() as launches:
                 logits = self.model.forward(self.context(arena, shape, padded=False))
+        if self.workspace.moved != moved:
+            # a buffer was replaced by a larger one inside this pass: launches recorded before that hold
+            # the old address.  The shape's next coming, which finds every buffer in place, records the plan.
+            entry.plan = None
+            return logits
         entry.plan, entry.plan_arena = LaunchPlan(launches), arena
         entry.plan_generation, entry.plan_logits = self.workspace.generation, logits
         return logits

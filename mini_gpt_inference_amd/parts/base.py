@@ -150,6 +150,7 @@ class Workspace:
         self._buffers: Dict[tuple, torch.Tensor] = {}
         self.frozen = False   # set while a HIP graph owns the addresses
         self.generation = 0   # counts (re)allocations: a graph captured before one holds stale addresses
+        self.moved = 0        # counts buffers that were replaced by larger ones: an address handed out before is stale
 
     def get(self, name: str, rows: int, cols: int, dtype: torch.dtype) -> torch.Tensor:
         # one buffer per (name, width, dtype): layers of different widths that use the same name
@@ -159,6 +160,8 @@ class Workspace:
         if buf is None or buf.shape[0] < rows:
             if self.frozen:
                 raise WorkspaceFrozen(f"workspace buffer {name!r} would have to grow while a graph holds it")
+            if buf is not None:
+                self.moved += 1
             buf = torch.empty((rows, cols), dtype=dtype, device=self.device)
             self._buffers[key] = buf
             self.generation += 1

@@ -195,7 +195,8 @@ class SandwichNorm(Arrangement):
             self._check(parts)
         n, ws, B = ctx.n_rows, ctx.workspace, self.branches
         norm1 = parts["norm1"]
-        flat = ws.get("sublayer_sums", B * n, self.width, torch.float32)[:B * n]
+        # (a buffer per number of branches: one that grew from layer to layer inside a step would move)
+        flat = ws.get(f"sublayer_sums_{B}", B * n, self.width, torch.float32)[:B * n]
         ys = flat.view(B, n, self.width)
         h = ws.get("normed", n, self.width, ctx.dtype)
         norm1.forward(ctx, x, h, n, zero=flat.view(n, B * self.width))
