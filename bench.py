@@ -292,23 +292,53 @@ def viperax_like(layers, width, heads, vocab, window=512, streams=2):
             "embedding": {"scale": float(width) ** 0.5}, "logit_scale": 1.0, "logit_softcap": 30.0, "layers": out}
 
 
+def bobevik_like(layers, width, heads, vocab):
+    """A Bobevik config.json of a GPT-2-style model's size: the same layers, width and vocabulary, heads of
+    128 channels; the layer types in turn (parallel, retention, attention, retention; two layers: parallel,
+    attention); every token goes through 8 width^2 feed-forward elements a layer, as through the GPT-2 MLP
+    (a gated unit with a hidden size of 8/3 width).  Attention layers have a quarter as many key/value heads
+    as heads and mix values; a parallel layer gives half the heads to each side."""
+    ff = width * 8 // 3 // 64 * 64
+    kinds = ["parallel", "attention"] if layers <= 2 else ["parallel", "retention", "attention", "retention"]
+    out = []
+    for i in range(layers):
+        kind = kinds[i % len(kinds)]
+        if kind == "retention":
+            mixer = {"heads": heads, "dim": 128, "vdim": 128, "decay": [1.0 - 2.0 ** (-5 - h % 8) for h in range(heads)],
+                     "rot": {"dims": 64, "base": 1e6}}
+        elif kind == "attention":
+            mixer = {"heads": heads, "kv_heads": max(heads // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                     "rot": {"dims": 128, "base": 10000.0}, "v_mix": True}
+        else:
+            half = max(heads // 2, 1)
+            mixer = {"left": {"heads": half, "kv_heads": max(half // 4, 1), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "rot": {"dims": 64, "base": 50000.0, "scaling": {"factor": 4.0}}, "softcap": 30.0},
+                     "right": {"heads": half, "dim": 128, "vdim": 128,
+                               "decay": [1.0 - 2.0 ** (-1 - h % 10) for h in range(half)]}}
+        out.append({"type": kind, "mixer": mixer, "mlp": {"kind": "dense", "ff": ff}})
+    return {"architecture": "Bobevik", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+            "layers": out}
+
+
+COMPARED = {"viperax": viperax_like, "bobevik": bobevik_like}
+
+
 def compare_run(args, name):
-    """--compare viperax: prefill (2 prompts of 1,024 tokens as one step) and decode (batch 8, by the
-    default run's timing rule, fewer blocks) of Viperax beside the GPT-2-style model at equal layers,
-    width, heads and vocabulary, random weights, at COMPARE_SIZES.  One JSON line."""
+    """--compare viperax | bobevik: prefill (2 prompts of 1,024 tokens as one step) and decode (batch 8,
+    by the default run's timing rule, fewer blocks) of that design beside the GPT-2-style model at equal
+    layers, width, heads and vocabulary, random weights, at COMPARE_SIZES.  One JSON line."""
     import argparse as _argparse
     import gc
 
     import torch
 
-    assert name == "viperax"
     vocab, rows = 32768, []
     for layers, width, heads in COMPARE_SIZES:
         row = {"layers": layers, "width": width, "heads": heads, "vocab": vocab}
         for label, raw in (("gpt2-mini", {"architecture": "gpt2-mini", "n_layer": layers, "n_embd": width,
                                           "n_head": heads, "vocab_size": vocab, "block_size": args.positions,
                                           "bias": True, "layer_norm_eps": 1e-5}),
-                           ("viperax", viperax_like(layers, width, heads, vocab))):
+                           (name, COMPARED[name](layers, width, heads, vocab))):
             a = _argparse.Namespace(**vars(args))
             a.raw_config = raw
             pre = prefill_run(a, args.dtype, reps=10, warmups=5)
@@ -328,7 +358,7 @@ def compare_run(args, name):
             torch.cuda.empty_cache()
         rows.append(row)
         print(f"[bench] compared {row}", file=sys.stderr, flush=True)
-    return {"compare": "viperax beside gpt2-mini at equal layers, width, heads and vocabulary", "dtype": args.dtype,
+    return {"compare": f"{name} beside gpt2-mini at equal layers, width, heads and vocabulary", "dtype": args.dtype,
             "batch": args.batch, "prompt_len": args.prompt, "prefill": "2 x 1024 tokens, one step", "rows": rows}
 
 
@@ -436,7 +466,7 @@ def main(argv=None) -> int:
                          "commit and the software and device that ran them")
     ap.add_argument("--prefill-requests", type=int, default=2,
                     help="prompts of 1,024 tokens in the prefill step (the default run's 2,048 tokens are 2)")
-    ap.add_argument("--compare", choices=["viperax"], default=None,
+    ap.add_argument("--compare", choices=sorted(COMPARED), default=None,
                     help="prefill and decode of that design beside the GPT-2-style model at equal sizes (COMPARE_SIZES)")
     ap.add_argument("--prefill-only", action="store_true",
                     help="run only the 2,048-token prefill and print its record (for profiling)")

@@ -24,7 +24,8 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
-    int n_kv_head, int head_dim, int page_size, float scale, int window, const float* __restrict__ sinks) {
+    int n_kv_head, int head_dim, int page_size, float scale, int window, const float* __restrict__ sinks,
+    float softcap) {
   __shared__ float q_s[AD_MAX_DPL * 64];
   __shared__ float p_s[AD_WAVES][64];
   __shared__ int page_s[AD_WAVES][64];
@@ -73,7 +74,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
           dot = fmaf(q_s[d + 2 * e + 1], __uint_as_float(w[e] & 0xffff0000u), dot);
         }
       }
-      s = dot;
+      s = softcap > 0.f ? softcap * tanh_fast(dot * __builtin_amdgcn_rcpf(softcap)) : dot;
     }
     const float m_new = fmaxf(m, wave_max(s));
     const float p = valid ? __expf(s - m_new) : 0.f;
@@ -143,7 +144,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, hipStream_t stream) {
+    const float* sinks, float softcap, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
@@ -153,7 +154,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
   hipLaunchKernelGGL(paged_attention_split_kernel, dim3(n_tokens, n_head), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,
                      block_tables, max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim,
-                     page_size, scale, window, sinks);
+                     page_size, scale, window, sinks, softcap);
   return mgpt_last_error();
 }
 
@@ -169,7 +170,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
-    int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks) {
+    int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks, float softcap) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   __shared__ float m_s[AD_WAVES], l_s[AD_WAVES];
@@ -238,6 +239,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
       }
 #pragma unroll
       for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, 64);
+      if (softcap > 0.f) dot = softcap * tanh_fast(dot * __builtin_amdgcn_rcpf(softcap));
       s[i] = valid[i] ? dot : -INFINITY;
       cmax = fmaxf(cmax, s[i]);
     }
@@ -296,7 +298,7 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, hipStream_t stream) {
+    const float* sinks, float softcap, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
@@ -307,7 +309,7 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
 #define AD_LAUNCH(DD)                                                                                   \
   hipLaunchKernelGGL(paged_attention_split_fast_kernel<DD>, grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,       \
-                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks)
+                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks, softcap)
   switch (head_dim) {
     case 16: AD_LAUNCH(16); break;
     case 32: AD_LAUNCH(32); break;

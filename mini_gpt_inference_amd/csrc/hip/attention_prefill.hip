@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_head, int n_kv_head, int page_size, float scale, int window,
-    int single_below, const float* __restrict__ sinks) {
+    int single_below, const float* __restrict__ sinks, float softcap) {
   constexpr int THREADS = 256 * G;
   constexpr int SB = PF_KT * G;    // keys staged per step
   // Key and value rows in LDS: as long as the head size where that is a power of two, the 16-byte
@@ -206,6 +206,14 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
 #pragma unroll
           for (int kt = 0; kt < NKT; ++kt)
             s[kt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kk][kt], qf[kk], s[kt], 0, 0, 0);
+      }
+      if (softcap > 0.f) {
+        // capped scores: cap * tanh(s * scale / cap), kept in the raw scores' units (times cap / scale)
+        const float in = scale * __builtin_amdgcn_rcpf(softcap), back = softcap * __builtin_amdgcn_rcpf(scale);
+#pragma unroll
+        for (int kt = 0; kt < NKT; ++kt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) s[kt][i] = back * tanh_fast(s[kt][i] * in);
       }
       // The value operands do not depend on the scores: asked for now, they arrive while the softmax
       // below keeps the wave busy.  k-slot (g, e) of operand (dt, bb): key bb*32 + g*4 + e for e < 4,
@@ -350,7 +358,7 @@ extern "C" int mgpt_prefill_attention_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req,
     int max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int single_below, const float* sinks, hipStream_t stream) {
+    int single_below, const float* sinks, float softcap, hipStream_t stream) {
   if (n_req == 0 || max_q_len == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens) return MGPT_ERR_NULL;
   if (n_req < 0 || max_q_len < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 ||
@@ -374,7 +382,7 @@ extern "C" int mgpt_prefill_attention_bf16(
     hipLaunchKernelGGL((prefill_attention_kernel<DD, GG>), grid, dim3(256 * GG), lds_bytes, stream,             \
                        (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,    \
                        block_tables, max_blocks, cu_q, seq_lens, n_head, n_kv_head, page_size, scale, window,   \
-                       single_below, sinks);                                                                          \
+                       single_below, sinks, softcap);                                                                          \
   }
   // Two wave groups halve the walk of a tile over its keys; one group leaves LDS for a second
   // workgroup on the compute unit.  The first serves a step with few tiles, the second one with many.

@@ -107,4 +107,10 @@ __device__ __forceinline__ float gelu_tanh_fast(float u) {
   return 0.5f * u * (1.0f + t);
 }
 
+// tanh(z) = 1 - 2 / (exp(2z) + 1) on the hardware's exp2 and reciprocal (a few ulp of float32; the ends are right)
+__device__ __forceinline__ float tanh_fast(float z) {
+  const float e = __builtin_amdgcn_exp2f(z * 2.8853900817779268f);
+  return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+}
+
 static inline int mgpt_last_error() { return (int)hipGetLastError(); }

@@ -156,3 +156,171 @@ extern "C" int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, i
 #undef DS_LAUNCH
   return mgpt_last_error();
 }
+
+// ---------------------------------------------------------------------------------------------
+// Prompt portions: the same recurrence a chunk of 32 tokens at a time, as matrix products on the
+// float32 matrix cores (v_mfma_f32_16x16x4_f32: true 32-bit products and sums).  For a chunk whose
+// tokens have in-chunk indices i = 0 .. n-1, with L = decay:
+//   P[i][j] = (q_i . k_j) L^(i-j) for j <= i, else 0
+//   o_i     = sum_j P[i][j] v_j + L^(i+1) S^T q_i
+//   S      <- L^n S + sum_j L^(n-1-j) k_j v_j^T
+// A workgroup owns (request, head, 32 value channels): the columns of S are independent of each
+// other, so a head's value channels are dealt out over workgroups, each of which makes P for itself.
+// Queries and keys come ready (activation, rotation, scale) as float32 from state_inputs_kernel.
+
+#define DC_C 32        // tokens a chunk
+#define DC_EB 32       // value channels a workgroup
+#define DC_DMAX 128    // largest head size of this path
+#define DC_LDQ (DC_DMAX + 4)
+#define DC_LDE (DC_EB + 4)
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void state_inputs_kernel(const void* __restrict__ z, int dtype, long ldz, int q_off,
+                                                           int k_off, int n_head, int D, int act,
+                                                           const int* __restrict__ positions, const float* __restrict__ freq,
+                                                           int rot_dims, float k_scale, float* __restrict__ qk, int n_tokens) {
+  __shared__ float cos_s[DS_MAX / 2], sin_s[DS_MAX / 2];
+  const int n = blockIdx.x, half = rot_dims / 2;
+  if (freq) {
+    const float p = (float)positions[n];
+    for (int i = threadIdx.x; i < half; i += 256) {
+      const float a = p * freq[i];
+      cos_s[i] = cosf(a);
+      sin_s[i] = sinf(a);
+    }
+  }
+  __syncthreads();
+  const int HD = n_head * D;
+  float* dst = qk + (long)n * 2 * HD;
+  // thread: one channel of one head; a rotated pair is made by the thread of its first channel
+  for (int i = threadIdx.x; i < HD; i += 256) {
+    const int d = i % D;
+    if (d >= half && d < rot_dims) continue;
+    const long at = (long)n * ldz + i;
+    float q = ds_act(load_f(z, dtype, at + q_off), act), k = ds_act(load_f(z, dtype, at + k_off), act);
+    if (d < half) {
+      const float q2 = ds_act(load_f(z, dtype, at + half + q_off), act), k2 = ds_act(load_f(z, dtype, at + half + k_off), act);
+      const float co = cos_s[d], si = sin_s[d];
+      dst[i + half] = q2 * co + q * si;
+      dst[HD + i + half] = (k2 * co + k * si) * k_scale;
+      const float qr = q * co - q2 * si, kr = k * co - k2 * si;
+      q = qr;
+      k = kr;
+    }
+    dst[i] = q;
+    dst[HD + i] = k * k_scale;
+  }
+}
+
+__global__ __launch_bounds__(256) void decay_state_chunk_kernel(
+    const float* __restrict__ qk, const void* __restrict__ z, int dtype, long ldz, int v_off, int n_head, int D, int E,
+    int act, const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ state,
+    const int* __restrict__ state_slots, const int* __restrict__ cu_q, float* __restrict__ out, long ldo) {
+  __shared__ float Qs[DC_C][DC_LDQ], Ks[DC_C][DC_LDQ], Ss[DC_DMAX][DC_LDE], Vs[DC_C][DC_LDE], Ps[DC_C][DC_LDE];
+  __shared__ float pw[DC_C + 1];
+  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * DC_EB, tid = threadIdx.x;
+  const int slot = state_slots[r];
+  const int t_begin = cu_q[r], t_end = cu_q[r + 1];
+  if (slot < 0 || t_end <= t_begin) return;     // a request of the padding
+  const int wave = tid >> 6, lane = tid & 63, r16 = lane & 15, g = lane >> 4;
+  const int Dp = (D + 15) & ~15;                // rows of S and steps along d, padded with zeros
+  const int HD = n_head * D;
+  const float lambda = decay[h];
+  const float log_l = logf(lambda);
+  if (tid <= DC_C) pw[tid] = tid == 0 ? 1.0f : expf((float)tid * log_l);
+  float* st = state + ((long)slot * n_head + h) * (long)D * E;
+  const bool fresh = positions[t_begin] == 0;
+  for (int i = tid; i < Dp * DC_EB; i += 256) {
+    const int d = i / DC_EB, c = i - d * DC_EB;
+    Ss[d][c] = (!fresh && d < D && e0 + c < E) ? st[(long)d * E + e0 + c] : 0.f;
+  }
+  const int ti = wave >> 1, tj = wave & 1;      // this wave's 16 x 16 tile of P and of the chunk's outputs
+
+  for (int t0 = t_begin; t0 < t_end; t0 += DC_C) {
+    const int nt = t_end - t0 < DC_C ? t_end - t0 : DC_C;
+    __syncthreads();     // the chunk before is done with the staged rows; S is whole
+    for (int i = tid; i < DC_C * Dp; i += 256) {
+      const int tt = i / Dp, d = i - tt * Dp;
+      const bool ok = tt < nt && d < D;
+      const long at = (long)(t0 + tt) * 2 * HD + (long)h * D + d;
+      Qs[tt][d] = ok ? qk[at] : 0.f;
+      Ks[tt][d] = ok ? qk[at + HD] : 0.f;
+    }
+    for (int i = tid; i < DC_C * DC_EB; i += 256) {
+      const int tt = i / DC_EB, c = i - tt * DC_EB;
+      Vs[tt][c] = (tt < nt && e0 + c < E)
+                      ? ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + e0 + c), act) : 0.f;
+    }
+    __syncthreads();
+    // ---- P = Q K^T with the decay of the distance, lower triangle
+    {
+      f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+      if (tj <= ti) {
+        for (int k0 = 0; k0 < Dp; k0 += 4)
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ks[tj * 16 + r16][k0 + g], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int i = ti * 16 + 4 * g + v, j = tj * 16 + r16;
+        Ps[i][j] = j <= i ? acc[v] * pw[i - j] : 0.f;
+      }
+    }
+    __syncthreads();
+    // ---- o = P V + L^(i+1) Q S
+    {
+      f32x4_t a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
+      for (int k0 = 0; k0 < (ti + 1) * 16; k0 += 4)
+        a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[ti * 16 + r16][k0 + g], Vs[k0 + g][tj * 16 + r16], a1, 0, 0, 0);
+      for (int k0 = 0; k0 < Dp; k0 += 4)
+        a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ss[k0 + g][tj * 16 + r16], a2, 0, 0, 0);
+#pragma unroll
+      for (int v = 0; v < 4; ++v) {
+        const int i = ti * 16 + 4 * g + v, c = e0 + tj * 16 + r16;
+        if (i < nt && c < E) out[(long)(t0 + i) * ldo + (long)h * E + c] = a1[v] + pw[i + 1] * a2[v];
+      }
+    }
+    __syncthreads();     // every wave has read the old S
+    // ---- S <- L^n S + sum_t L^(n-1-t) k_t v_t^T: the tiles (di, tj) with di = ti, ti + 2, ...
+    for (int di = ti; di * 16 < Dp; di += 2) {
+      f32x4_t acc;
+#pragma unroll
+      for (int v = 0; v < 4; ++v) acc[v] = pw[nt] * Ss[di * 16 + 4 * g + v][tj * 16 + r16];
+      for (int k0 = 0; k0 < DC_C; k0 += 4) {
+        const int t = k0 + g;
+        const float w = t < nt ? pw[nt - 1 - t] : 0.f;
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[t][di * 16 + r16] * w, Vs[t][tj * 16 + r16], acc, 0, 0, 0);
+      }
+#pragma unroll
+      for (int v = 0; v < 4; ++v) Ss[di * 16 + 4 * g + v][tj * 16 + r16] = acc[v];
+    }
+  }
+  __syncthreads();
+  for (int i = tid; i < D * DC_EB; i += 256) {
+    const int d = i / DC_EB, c = i - d * DC_EB;
+    if (e0 + c < E) st[(long)d * E + e0 + c] = Ss[d][c];
+  }
+}
+
+// The chunked form for steps with prompt portions: qk is scratch, float32 [n_tokens, 2 * n_head * head_dim]; out is
+// float32 [n_tokens, >= n_head * value_dim]: the heads' raw outputs (norm and gate are the caller's next kernel).
+// Head sizes up to 128 (value sizes up to 256); others are refused with MGPT_ERR_BAD_SHAPE and nothing launched.
+extern "C" int mgpt_decay_state_chunked(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int n_head,
+                                        int head_dim, int value_dim, int act, const int* positions, const float* freq,
+                                        int rot_dims, float k_scale, const float* decay, float* state,
+                                        const int* state_slots, const int* cu_q, int n_req, int n_tokens, float* qk,
+                                        float* out, long ldo, hipStream_t stream) {
+  if (n_req == 0 || n_tokens == 0) return MGPT_OK;
+  if (!z || !positions || !decay || !state || !state_slots || !cu_q || !out || !qk) return MGPT_ERR_NULL;
+  if (!dtype_ok(dtype)) return MGPT_ERR_BAD_DTYPE;
+  const int D = head_dim, E = value_dim;
+  if (n_req < 0 || n_tokens < 0 || n_head <= 0 || D <= 0 || E <= 0 || D > DC_DMAX || E > DS_MAX || rot_dims < 0 ||
+      (rot_dims & 1) || rot_dims > D || (act != 0 && act != 1))
+    return MGPT_ERR_BAD_SHAPE;
+  if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
+  hipLaunchKernelGGL(state_inputs_kernel, dim3(n_tokens), dim3(256), 0, stream, z, dtype, ldz, q_off, k_off, n_head, D, act,
+                     positions, rot_dims ? freq : nullptr, rot_dims, k_scale, qk, n_tokens);
+  hipLaunchKernelGGL(decay_state_chunk_kernel, dim3(n_req, n_head, (E + DC_EB - 1) / DC_EB), dim3(256), 0, stream, qk, z,
+                     dtype, ldz, v_off, n_head, D, E, act, positions, decay, state, state_slots, cu_q, out, ldo);
+  return mgpt_last_error();
+}

@@ -30,29 +30,40 @@ __device__ __forceinline__ float rms_gate_act(float g, int act) {
   return g;
 }
 
-// one wave per segment
+// sum over the workgroup's threads (1, 2 or 4 waves), the same value in every thread; waves are added in order
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  if (blockDim.x == 64) return v;
+  const int wave = threadIdx.x >> 6;
+  __syncthreads();      // the scratch's readers of the call before are done
+  if ((threadIdx.x & 63) == 0) scratch[wave] = v;
+  __syncthreads();
+  return blockDim.x == 128 ? scratch[0] + scratch[1] : (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
+}
+
+// one workgroup per segment: a wave for a narrow one (a head), four for a wide one (a row of the model's width)
 __global__ __launch_bounds__(256) void rms_norm_kernel(
     const void* __restrict__ x, int x_dtype, long ldx, const int* __restrict__ rows,
     const float* __restrict__ gain, float offset, float eps, float mult, const void* __restrict__ gate,
     int gate_dtype, long ldg, int gate_act, void* out, int out_dtype, long ldo, int accumulate,
     float* __restrict__ zero, long ldz, int zero_width, int n_rows, int groups, int x_gstride, int o_gstride,
     int width) {
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const long seg = (long)blockIdx.x * 4 + wave;
-  if (seg >= (long)n_rows * groups) return;
+  __shared__ float scratch[4];
+  const long seg = blockIdx.x;
   const int row = (int)(seg / groups), g = (int)(seg - (long)row * groups);
   const int src = rows ? rows[row] : row;
   const long xb = (long)src * ldx + (long)g * x_gstride;
+  const int step = blockDim.x;
   float ss = 0.f;
-  for (int c = lane; c < width; c += 64) {
+  for (int c = threadIdx.x; c < width; c += step) {
     const float v = load_f(x, x_dtype, xb + c);
     ss = fmaf(v, v, ss);
   }
-  ss = wave_sum(ss);
+  ss = block_sum(ss, scratch);
   const float r = mult / sqrtf(ss / (float)width + eps);
   const long ob = (long)row * ldo + (long)g * o_gstride;
   const long gb = (long)row * ldg + (long)g * o_gstride;
-  for (int c = lane; c < width; c += 64) {
+  for (int c = threadIdx.x; c < width; c += step) {
     float v = load_f(x, x_dtype, xb + c) * r;
     if (gain) v *= offset + gain[(long)g * width + c];
     if (gate) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), gate_act);
@@ -60,7 +71,7 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
     store_f(out, out_dtype, ob + c, v);
   }
   if (zero && g == 0)
-    for (int c = lane; c < zero_width; c += 64) zero[(long)row * ldz + c] = 0.f;
+    for (int c = threadIdx.x; c < zero_width; c += step) zero[(long)row * ldz + c] = 0.f;
 }
 
 extern "C" int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* rows, const float* gain, float offset,
@@ -73,8 +84,9 @@ extern "C" int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* ro
   if (n_rows < 0 || groups <= 0 || width <= 0 || zero_width < 0) return MGPT_ERR_BAD_SHAPE;
   if (!dtype_ok(x_dtype) || !dtype_ok(out_dtype) || (gate && !dtype_ok(gate_dtype))) return MGPT_ERR_BAD_DTYPE;
   const long segs = (long)n_rows * groups;
-  if (segs > (1L << 32)) return MGPT_ERR_TOO_LARGE;
-  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)((segs + 3) / 4)), dim3(256), 0, stream, x, x_dtype, ldx, rows,
+  if (segs > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
+  const int threads = width <= 256 ? 64 : (width <= 512 ? 128 : 256);
+  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)segs), dim3(threads), 0, stream, x, x_dtype, ldx, rows,
                      gain, offset, eps, mult, gate, gate_dtype, ldg, gate_act, out, out_dtype, ldo, accumulate, zero,
                      ldz, zero_width, n_rows, groups, x_gstride, o_gstride, width);
   return mgpt_last_error();

@@ -486,7 +486,8 @@ def linear_skinny_partials(n_rows: int, n_out: int, k_dim: int, has_ln: bool, ep
 def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                                block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                                q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
-                               window: int = 0, fast: bool = True, sinks: Optional[torch.Tensor] = None) -> bool:
+                               window: int = 0, fast: bool = True, sinks: Optional[torch.Tensor] = None,
+                               softcap: float = 0.0) -> bool:
     """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused.
     fast=False keeps to the variant that takes every head size."""
     if q.dtype != torch.bfloat16:
@@ -502,7 +503,7 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
     rc = fn(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _ptr(sinks), _stream())
+        page_size, float(scale), int(window), _ptr(sinks), float(softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_split_bf16")
@@ -513,7 +514,7 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
                                 block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor,
                                 n_tokens: int, n_head: int, scale: float, window: int = 0,
                                 identity: bool = False, cu_q: Optional[torch.Tensor] = None,
-                                sinks: Optional[torch.Tensor] = None) -> bool:
+                                sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> bool:
     """bfloat16 attention for single tokens (one query per request and step), keys split over eight
     waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
     padded token; identity=True promises q_req[n] in (n, -1).  With cu_q (the requests' token offsets;
@@ -548,7 +549,7 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     rc = library.kernels().mgpt_paged_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(positions), _ptr(q_req), _ptr(cu_q), n_tokens, n_head, n_kv_head, head_dim, page_size,
-        num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), _stream())
+        num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), float(softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_decode_bf16")
@@ -658,7 +659,7 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
                            max_q_len: int, n_head: int, scale: float, window: int = 0,
-                           single_below: int = 0, sinks: Optional[torch.Tensor] = None) -> bool:
+                           single_below: int = 0, sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> bool:
     """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
     rows of q from cu_q; a request may bring none).  Requests that bring exactly one token, and that
     among the step's first `single_below` tokens, are left to another kernel.  False when it does
@@ -685,7 +686,7 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
     rc = library.kernels().mgpt_prefill_attention_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), int(single_below), _ptr(sinks), _stream())
+        page_size, float(scale), int(window), int(single_below), _ptr(sinks), float(softcap), _stream())
     if rc == -2:
         return False
     _check(rc, "prefill_attention_bf16")
@@ -1396,3 +1397,42 @@ def decay_state(z: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int,
         _ptr(positions), _ptr(freq), rot_dims, float(k_scale), _ptr(decay), _ptr(state), _ptr(state_slots), _ptr(cu_q),
         n_req, -1.0 if norm_eps is None else float(norm_eps), _ptr(out), _dtype_code(out), out.stride(0), _stream())
     _check(rc, "decay_state")
+
+
+CHUNKED_STATE_MAX_DIM = 128     # largest head size that the chunked form of the decaying state takes
+
+
+def decay_state_chunked(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int, head_dim: int, value_dim: int,
+                        decay: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor, cu_q: torch.Tensor,
+                        n_req: int, n_tokens: int, positions: torch.Tensor, qk: torch.Tensor, out: torch.Tensor,
+                        silu_inputs: bool = False, freq: Optional[torch.Tensor] = None, k_scale: float = 1.0) -> bool:
+    """decay_state for steps with prompt portions: the recurrence 32 tokens at a time as float32 matrix products.
+    out: float32 rows, the heads' raw outputs (no norm, no gate); qk: float32 scratch [>= n_tokens, 2 * heads * dim].
+    False, with nothing launched, for head sizes beyond CHUNKED_STATE_MAX_DIM."""
+    if head_dim > CHUNKED_STATE_MAX_DIM:
+        return False
+    _need_cuda(z, decay, state, state_slots, cu_q, positions, out, freq, qk)
+    _rows_2d("decay_state z", z, n_tokens)
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.stride(1) == 1 and out.shape[0] >= n_tokens
+          and out.shape[1] >= n_head * value_dim, "decay_state_chunked: out must be float32 rows of all heads' values")
+    _need(qk.dtype == torch.float32 and qk.is_contiguous() and qk.shape[0] >= n_tokens
+          and qk.shape[1] == 2 * n_head * head_dim, "decay_state_chunked: qk must be float32 [tokens, 2 * heads * dim]")
+    _need(z.shape[1] >= max(q_off, k_off) + n_head * head_dim and z.shape[1] >= v_off + n_head * value_dim,
+          "decay_state_chunked: z is too narrow")
+    _need(decay.dtype == torch.float32 and decay.numel() == n_head, "decay_state: one float32 decay per head")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.is_contiguous()
+          and state.shape[1] == n_head * head_dim * value_dim, "decay_state: state must be [slots, heads * dim * vdim] float32")
+    _need_i32("state_slots", state_slots, n_req)
+    _need_i32("cu_q", cu_q, n_req + 1)
+    _need_i32("positions", positions, n_tokens)
+    _need(0 < value_dim <= 256, "decay_state takes value sizes up to 256")
+    rot_dims = 0
+    if freq is not None:
+        _need(freq.dtype == torch.float32 and freq.is_contiguous() and 2 * freq.numel() <= head_dim, "decay_state: bad frequencies")
+        rot_dims = 2 * freq.numel()
+    rc = library.kernels().mgpt_decay_state_chunked(
+        _ptr(z), _dtype_code(z), z.stride(0), q_off, k_off, v_off, n_head, head_dim, value_dim, int(silu_inputs),
+        _ptr(positions), _ptr(freq), rot_dims, float(k_scale), _ptr(decay), _ptr(state), _ptr(state_slots), _ptr(cu_q),
+        n_req, n_tokens, _ptr(qk), _ptr(out), out.stride(0), _stream())
+    _check(rc, "decay_state_chunked", 2)
+    return True

@@ -127,15 +127,15 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
         "mgpt_linear_skinny_row_groups": [I, I, I],
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
-        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P],
-        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, P],
-        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, P],
+        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P],
+        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P],
+        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
         "mgpt_linear_mfma_parts": [P, L, P, P, P, L, I, I, I, P],
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
-        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, P],
+        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, F, P],
         # a residual that is still a sum: base, partials, n_parts, part_stride, token table, position table, ids, positions
         "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
                                         I, I, I, I, I, I, F, P],
@@ -165,6 +165,7 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, P],
         "mgpt_head_gate": [P, I, L, I, I, P, I, L, I, I, P],
         "mgpt_decay_state": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, F, P, I, L, P],
+        "mgpt_decay_state_chunked": [P, I, L, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, P, P, L, P],
         "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, P, I, I, I, P],
         "mgpt_gather_rows": [P, L, P, P, L, I, I, P],
         "mgpt_linear_mfma_grouped": [P, L, P, L, P, P, I, P, I, L, I, I, I, P],

@@ -459,14 +459,29 @@ class DecayStateMixer(Mixer):
         z = ws.get("decay_state_in", n, self.in_weight.shape[0], ctx.dtype)
         linear(ctx, h, self.in_weight, None, z, n)
         y = ws.get("decay_state_out", n, self.v_width, ctx.dtype)
-        gated_here = self.head_norm_eps is not None
-        o = y if gated_here else ws.get("decay_state_sums", n, self.v_width, torch.float32)
-        kernels.decay_state(z, 0, self.k_off, self.v_off, self.g_off if gated_here else -1, self.n_head, self.head_dim,
-                            self.value_dim, self._decays(z.device), ctx.state_pools[binding.index], ctx.state_slots,
-                            ctx.cu_q, ctx.cu_q.numel() - 1, ctx.positions, o, silu_inputs=self.silu_inputs,
-                            freq=self.rotation.frequencies(z.device) if self.rotation is not None else None,
-                            k_scale=self.k_scale, norm_eps=self.head_norm_eps)
-        if not gated_here:
-            kernels.rms_norm(o, self.norm_weight, y, n, self.out_norm_eps, self.v_width, gate=z[:, self.g_off:],
+        freq = self.rotation.frequencies(z.device) if self.rotation is not None else None
+        state, n_req = ctx.state_pools[binding.index], ctx.cu_q.numel() - 1
+        # a step with prompt portions: the recurrence a chunk of tokens at a time on the matrix cores, the
+        # heads' norm and gate in a kernel behind it; single tokens: token by token, norm and gate inside
+        chunked = False
+        if not ctx.decode_only and self.head_dim <= kernels.CHUNKED_STATE_MAX_DIM:
+            sums = ws.get("decay_state_sums", n, self.v_width, torch.float32)
+            qk = ws.get("decay_state_qk", n, 2 * self.qk_width, torch.float32)
+            chunked = kernels.decay_state_chunked(z, 0, self.k_off, self.v_off, self.n_head, self.head_dim, self.value_dim,
+                                                  self._decays(z.device), state, ctx.state_slots, ctx.cu_q, n_req, n,
+                                                  ctx.positions, qk, sums, silu_inputs=self.silu_inputs, freq=freq,
+                                                  k_scale=self.k_scale)
+        gated_inside = self.head_norm_eps is not None and not chunked
+        if not chunked:
+            sums = y if gated_inside else ws.get("decay_state_sums", n, self.v_width, torch.float32)
+            kernels.decay_state(z, 0, self.k_off, self.v_off, self.g_off if gated_inside else -1, self.n_head,
+                                self.head_dim, self.value_dim, self._decays(z.device), state, ctx.state_slots, ctx.cu_q,
+                                n_req, ctx.positions, sums, silu_inputs=self.silu_inputs, freq=freq, k_scale=self.k_scale,
+                                norm_eps=self.head_norm_eps)
+        if self.head_norm_eps is not None and not gated_inside:
+            kernels.rms_norm(sums, None, y, n, self.head_norm_eps, self.value_dim, groups=self.n_head,
+                             gate=z[:, self.g_off:], gate_act="silu")
+        elif self.head_norm_eps is None:
+            kernels.rms_norm(sums, self.norm_weight, y, n, self.out_norm_eps, self.v_width, gate=z[:, self.g_off:],
                              gate_act="sigmoid")
         linear_add(ctx, y, self.out_weight, None, x, n)

@@ -130,6 +130,7 @@ class ModelCost:
     run_matrix_elements: int      # matrix elements a token goes through in the layers, over all runs of the order
     head_matrix_elements: int     # matrix elements a wanted logit row goes through behind the last run
     kv_runs: Tuple[KVRun, ...]    # every (run, mixer) that reads keys and values, its own cache or another run's
+    state_floats: int = 0         # float32 values of per-request state that a token's step reads (and writes), over all runs
 
     def step_read_bytes(self, n_tokens: int, context_lens, cache_itemsize: int) -> float:
         """Bytes that a step of n_tokens single tokens has to read when request i has context_lens[i]
@@ -140,7 +141,7 @@ class ModelCost:
             for c in context_lens:
                 reach = min(c, run.window) if run.window else c
                 kv += reach * run.tensors * run.n_kv_head * run.head_dim * cache_itemsize
-        return self.whole_tensor_bytes + n_tokens * self.table_row_bytes + kv
+        return self.whole_tensor_bytes + n_tokens * self.table_row_bytes + kv + 4.0 * self.state_floats * len(context_lens)
 
     def prompt_flops(self, prompt_lens, n_logit_rows: int) -> float:
         """Multiply-adds times two of whole prompts in one step: the matrices for every token, causal
@@ -273,7 +274,7 @@ class DecoderModel:
                     total += n
             return total
 
-        run_elements, kv_runs = 0, []
+        run_elements, kv_runs, state_floats = 0, [], 0
         for run in self.spec.order:
             layer = self.layers[run.layer]
             for part in layer.parts.values():
@@ -282,8 +283,10 @@ class DecoderModel:
                 if isinstance(need, KVNeed):
                     kv_runs.append(KVRun(int(getattr(part, "n_head", need.n_kv_head)), need.n_kv_head,
                                          need.head_dim, need.window, 1 if need.joint else 2))
+                elif isinstance(need, StateNeed):
+                    state_floats += int(need.numel)
         return ModelCost(sum(size(name) for name in whole), row_bytes, run_elements, matrices(self.head),
-                         tuple(kv_runs))
+                         tuple(kv_runs), state_floats)
 
     # ------------------------------------------------------------------ cache
     def _plan_cache(self) -> CacheLayout:

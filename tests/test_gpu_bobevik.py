@@ -298,6 +298,82 @@ def test_decaying_state_whole_in_portions_and_slots_used_again(dtype, H, D, E):
         helpers.assert_close(state[1:4], whole_state[1:4], "float32", f"{variant} state")
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("H,D,E", [(2, 16, 24), (1, 64, 64), (2, 128, 128), (3, 20, 12), (1, 128, 200), (2, 8, 256),
+                                   (1, 1, 1), (1, 30, 33)])
+def test_decaying_state_a_chunk_at_a_time(dtype, H, D, E):
+    """The matrix-core form for prompt portions against the plain recurrence: requests whose lengths are
+    below, at and beyond the chunk of 32 tokens, in one step; then cut into portions that end inside
+    chunks, beside single tokens, the states carried in slots poisoned before."""
+    g = torch.Generator().manual_seed(H * D + E + 1)
+    lens = [70, 1, 32, 33]
+    n = sum(lens)
+    z, k_off, v_off, g_off = _state_case(g, dtype, lens, H, D, E)
+    decay = torch.tensor([0.999, 0.6, 0.9][:H])
+    dims = D - D % 2 if D >= 2 else 0
+    for variant in ("rotated", "silu"):
+        f = P.silu if variant == "silu" else (lambda t: t)
+        want = torch.zeros(n, H * E, dtype=P.DTYPE)
+        at = 0
+        for T in lens:
+            rows = _d(z[at:at + T])
+            q, k = f(rows[:, :H * D]).view(T, H, D), f(rows[:, k_off:k_off + H * D]).view(T, H, D)
+            v = f(rows[:, v_off:v_off + H * E]).view(T, H, E)
+            if variant == "rotated":
+                if dims:
+                    q, k = P.rotate_half(q, dims, 1000.0), P.rotate_half(k, dims, 1000.0)
+                k = k * 0.25
+            want[at:at + T] = P.decaying_state(q, k, v, decay.tolist()).reshape(T, H * E)
+            at += T
+        freq = _freq(dims, 1000.0).to(DEV) if (variant == "rotated" and dims) else None
+
+        def run(steps, state, out):
+            for step in steps:
+                rows, pos, cu, slots = [], [], [0], []
+                for r, first, count in step:
+                    base = sum(lens[:r])
+                    rows += list(range(base + first, base + first + count))
+                    pos += list(range(first, first + count))
+                    cu.append(len(rows))
+                    slots.append(4 - r)
+                cu += [len(rows)] * 2
+                slots += [-1, 0]
+                zs = z[rows].to(DEV)
+                o = torch.zeros(len(rows), H * E, device=DEV)
+                qk = torch.zeros(len(rows), 2 * H * D, device=DEV)
+                assert kernels.decay_state_chunked(zs, 0, k_off, v_off, H, D, E, decay.to(DEV), state,
+                                                   torch.tensor(slots, dtype=torch.int32, device=DEV),
+                                                   torch.tensor(cu, dtype=torch.int32, device=DEV), len(slots), len(rows),
+                                                   torch.tensor(pos, dtype=torch.int32, device=DEV), qk, o,
+                                                   silu_inputs=variant == "silu", freq=freq,
+                                                   k_scale=0.25 if variant == "rotated" else 1.0)
+                out[rows] = o.cpu().to(P.DTYPE)
+
+        state = torch.full((6, H * D * E), float("nan"), device=DEV)
+        got = torch.zeros(n, H * E, dtype=P.DTYPE)
+        run([[(0, 0, 70), (1, 0, 1), (2, 0, 32), (3, 0, 33)]], state, got)
+        helpers.assert_close(got, want, "float32", f"{variant} whole")
+        assert torch.isnan(state[0]).all() and torch.isnan(state[5]).all() and torch.isfinite(state[1:5]).all()
+        whole_state = state.clone()
+        got2 = torch.zeros(n, H * E, dtype=P.DTYPE)
+        run([[(0, 0, 31), (3, 0, 2)], [(0, 31, 2), (1, 0, 1), (3, 2, 30)], [(3, 32, 1), (0, 33, 36), (2, 0, 17)],
+             [(0, 69, 1), (2, 17, 15)]], state, got2)
+        helpers.assert_close(got2, want, "float32", f"{variant} portions")
+        helpers.assert_close(state[1:5], whole_state[1:5], "float32", f"{variant} state")
+        # and the token-by-token kernel goes on from a state that the chunked one left
+        if variant == "silu":
+            extra = _rnd(g, 3, z.shape[1], dtype=dtype)
+            rows = _d(torch.cat([z[:70], extra]))
+            q, k = P.silu(rows[:, :H * D]).view(73, H, D), P.silu(rows[:, k_off:k_off + H * D]).view(73, H, D)
+            v = P.silu(rows[:, v_off:v_off + H * E]).view(73, H, E)
+            ref = P.decaying_state(q, k, v, decay.tolist()).reshape(73, H * E)[70:]
+            o = torch.zeros(3, H * E, device=DEV)
+            kernels.decay_state(extra.to(DEV), 0, k_off, v_off, -1, H, D, E, decay.to(DEV), state,
+                                torch.tensor([4], dtype=torch.int32, device=DEV), torch.tensor([0, 3], dtype=torch.int32, device=DEV),
+                                1, torch.tensor([70, 71, 72], dtype=torch.int32, device=DEV), o, silu_inputs=True)
+            helpers.assert_close(o, ref, "float32", "token by token behind chunks")
+
+
 def test_the_state_far_back_matters():
     """With a decay near one the first token's key and value are still in the output after hundreds
     of tokens (a lost or restarted state shows), with a fast decay they are gone."""
@@ -341,6 +417,47 @@ def test_capped_scores_in_attention_with_a_key_that_stands_out(dtype):
                                     perm.to(torch.int32).view(1, pages).to(DEV), i32([0, T - first]), i32([T]),
                                     i32([0] * (T - first)), T - first, 1, H, scale, softcap=cap)
     helpers.assert_close(out[:T - first], want[first:].reshape(T - first, H * D), dtype, "capped attention")
+
+
+@pytest.mark.parametrize("D", [32, 64, 128])
+def test_capped_scores_in_the_bfloat16_attention_kernels(D):
+    """The same construction through the matrix-core kernel for portions, the decode kernel and the
+    kernel that splits a query's keys over waves: the cap must bite in each."""
+    g = torch.Generator().manual_seed(7 + D)
+    H, G, page, T = 4, 2, 16, 208
+    q, k, v = _rnd(g, T, H, D, dtype="bfloat16"), _rnd(g, T, G, D, dtype="bfloat16"), _rnd(g, T, G, D, dtype="bfloat16")
+    far = 2 * page - 1
+    k[far] *= 4.0
+    q[-1] = k[far].float().repeat_interleave(H // G, dim=0).to(torch.bfloat16)
+    cap, scale = 3.0, D ** -0.5
+    want = P.causal_softmax_attention(_d(q), _d(k), _d(v), scale, cap)
+    assert float((want[-1] - P.causal_softmax_attention(_d(q), _d(k), _d(v), scale, None)[-1]).abs().max()) > 0.3
+    pages = T // page
+    perm = torch.randperm(pages, generator=g)
+    kp = torch.zeros(pages, G, page, D, dtype=torch.bfloat16)
+    vp = torch.zeros(pages, G, page, D, dtype=torch.bfloat16)
+    for j in range(T):
+        kp[perm[j // page], :, j % page], vp[perm[j // page], :, j % page] = k[j], v[j]
+    kp, vp, bt = kp.to(DEV), vp.to(DEV), perm.to(torch.int32).view(1, pages).to(DEV)
+    i32 = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    first = 100
+    n = T - first
+    qd = q[first:].reshape(n, H * D).to(DEV)
+    out = torch.zeros(n, H * D, dtype=torch.bfloat16, device=DEV)
+    assert kernels.prefill_attention_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), 1, n, H, scale, softcap=cap)
+    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "tile kernel")
+    out.zero_()
+    assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
+                                              softcap=cap)
+    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "split kernel")
+    out.zero_()
+    assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
+                                              fast=False, softcap=cap)
+    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "split kernel, general variant")
+    one = torch.zeros(1, H * D, dtype=torch.bfloat16, device=DEV)
+    assert kernels.paged_attention_decode_bf16(qd[n - 1:], one, kp, vp, bt, i32([T - 1]), i32([0]), 1, H, scale,
+                                               identity=True, softcap=cap)
+    helpers.assert_close(one, want[T - 1:].reshape(1, H * D), "bfloat16", "decode kernel")
 
 
 # ---------------------------------------------------------------- the model through the step function
