@@ -237,26 +237,52 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
   }
   const int ti = wave >> 1, tj = wave & 1;      // this wave's 16 x 16 tile of P and of the chunk's outputs
 
+  // A chunk's rows travel from memory into registers while the chunk before is multiplied: thread tid holds
+  // elements tid, tid + 256, ... of the chunk's [32, Dp] queries and keys and of its [32, 32] values.
+  constexpr int QK_PT = DC_C * DC_DMAX / 256, V_PT = DC_C * DC_EB / 256;
+  float q_r[QK_PT], k_r[QK_PT], v_r[V_PT];
+  auto fetch = [&](int t0) {
+    const int nt = t_end - t0 < DC_C ? t_end - t0 : DC_C;      // may be <= 0
+#pragma unroll
+    for (int u = 0; u < QK_PT; ++u) {
+      const int i = tid + u * 256, tt = i / Dp, d = i - tt * Dp;
+      const bool ok = i < DC_C * Dp && tt < nt && d < D;
+      const long at = (long)(t0 + tt) * 2 * HD + (long)h * D + d;
+      q_r[u] = ok ? qk[at] : 0.f;
+      k_r[u] = ok ? qk[at + HD] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < V_PT; ++u) {
+      const int i = tid + u * 256, tt = i / DC_EB, c = i - tt * DC_EB;
+      v_r[u] = (tt < nt && e0 + c < E)
+                   ? ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + e0 + c), act) : 0.f;
+    }
+  };
+  fetch(t_begin);
+
   for (int t0 = t_begin; t0 < t_end; t0 += DC_C) {
     const int nt = t_end - t0 < DC_C ? t_end - t0 : DC_C;
     __syncthreads();     // the chunk before is done with the staged rows; S is whole
-    for (int i = tid; i < DC_C * Dp; i += 256) {
-      const int tt = i / Dp, d = i - tt * Dp;
-      const bool ok = tt < nt && d < D;
-      const long at = (long)(t0 + tt) * 2 * HD + (long)h * D + d;
-      Qs[tt][d] = ok ? qk[at] : 0.f;
-      Ks[tt][d] = ok ? qk[at + HD] : 0.f;
+#pragma unroll
+    for (int u = 0; u < QK_PT; ++u) {
+      const int i = tid + u * 256, tt = i / Dp, d = i - tt * Dp;
+      if (i < DC_C * Dp) {
+        Qs[tt][d] = q_r[u];
+        Ks[tt][d] = k_r[u];
+      }
     }
-    for (int i = tid; i < DC_C * DC_EB; i += 256) {
-      const int tt = i / DC_EB, c = i - tt * DC_EB;
-      Vs[tt][c] = (tt < nt && e0 + c < E)
-                      ? ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + e0 + c), act) : 0.f;
+#pragma unroll
+    for (int u = 0; u < V_PT; ++u) {
+      const int i = tid + u * 256;
+      Vs[i / DC_EB][i % DC_EB] = v_r[u];
     }
     __syncthreads();
+    fetch(t0 + DC_C);     // (behind the last chunk: no token is left, nothing is loaded)
     // ---- P = Q K^T with the decay of the distance, lower triangle
     {
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       if (tj <= ti) {
+#pragma unroll 4
         for (int k0 = 0; k0 < Dp; k0 += 4)
           acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ks[tj * 16 + r16][k0 + g], acc, 0, 0, 0);
       }
@@ -270,8 +296,10 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     // ---- o = P V + L^(i+1) Q S
     {
       f32x4_t a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
       for (int k0 = 0; k0 < (ti + 1) * 16; k0 += 4)
         a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[ti * 16 + r16][k0 + g], Vs[k0 + g][tj * 16 + r16], a1, 0, 0, 0);
+#pragma unroll 4
       for (int k0 = 0; k0 < Dp; k0 += 4)
         a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ss[k0 + g][tj * 16 + r16], a2, 0, 0, 0);
 #pragma unroll
@@ -286,6 +314,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
       f32x4_t acc;
 #pragma unroll
       for (int v = 0; v < 4; ++v) acc[v] = pw[nt] * Ss[di * 16 + 4 * g + v][tj * 16 + r16];
+#pragma unroll
       for (int k0 = 0; k0 < DC_C; k0 += 4) {
         const int t = k0 + g;
         const float w = t < nt ? pw[nt - 1 - t] : 0.f;

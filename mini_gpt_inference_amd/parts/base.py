@@ -211,6 +211,9 @@ class StepContext:
     # a write into the residual streams that its arrangement has left to the next reader of the streams:
     # (mix, out, y) as for ops.kernels.streams_write; None: the streams are up to date
     pending_streams: Optional[Any] = None
+    # an addition to the residual that a layer has left to whoever reads the residual next (parts.block.PendingSandwich);
+    # None: the residual is up to date
+    pending_update: Optional[Any] = None
     # set by a caller that will choose greedily among the logits: an ops.linear.TileBest, which the
     # head fills beside the logits if its kernel can
     tile_best: Optional[Any] = None

@@ -190,25 +190,67 @@ class SandwichNorm(Arrangement):
             raise ValueError("the norms that join parallel mixers have plain gains")
         self._checked = True
 
+    # the arrangement reads ctx.pending_update: the addition that the layer before has left to be made
+    # together with this layer's first norm
+    takes_pending_update = True
+
+    def _buffers(self, ctx) -> torch.Tensor:
+        """[branches, rows, width] float32, zero: what the sublayers add their outputs into.  A buffer per number of
+        branches (one that grew from layer to layer inside a step would move); cleared when it is made, and by
+        the kernel that takes the sums out of it ever after."""
+        ws, n, B = ctx.workspace, ctx.n_rows, self.branches
+        made = ws.generation
+        flat = ws.get(f"sublayer_sums_{B}", B * n, self.width, torch.float32)
+        if ws.generation != made:
+            flat.zero_()
+        return flat[:B * n].view(B, n, self.width)
+
     def run(self, ctx, x, parts, bindings, position) -> None:
         if not self._checked:
             self._check(parts)
-        n, ws, B = ctx.n_rows, ctx.workspace, self.branches
+        n, B = ctx.n_rows, self.branches
         norm1 = parts["norm1"]
-        # (a buffer per number of branches: one that grew from layer to layer inside a step would move)
-        flat = ws.get(f"sublayer_sums_{B}", B * n, self.width, torch.float32)[:B * n]
-        ys = flat.view(B, n, self.width)
-        h = ws.get("normed", n, self.width, ctx.dtype)
-        norm1.forward(ctx, x, h, n, zero=flat.view(n, B * self.width))
+        ys = self._buffers(ctx)
+        h = ctx.workspace.get("normed", n, self.width, ctx.dtype)
+        left, ctx.pending_update = ctx.pending_update, None
+        if left is not None and left.goes_with(norm1, x, n):
+            left.run(norm1.weight, h)       # the layer before's last addition and this layer's first norm in one kernel
+        else:
+            if left is not None:
+                left.run(None, None)
+            norm1.forward(ctx, x, h, n)
         for b, role in enumerate(self.mixer_roles):
             parts[role].forward_add(ctx, h, ys[b], bindings[role], position)
         joins = [(ys[b], parts[self.join_roles[b]].weight if B > 1 else None) for b in range(B)]
-        norm1b = parts["norm1b"]
         if not self.has_feed_forward:
-            kernels.rms_post_norm(joins, x, norm1b.weight, n, norm1b.eps, norm1b.offset, self.mult)
+            ctx.pending_update = PendingSandwich(joins, x, parts["norm1b"], self.mult, n)
             return
+        norm1b = parts["norm1b"]
         kernels.rms_post_norm(joins, x, norm1b.weight, n, norm1b.eps, norm1b.offset, self.mult,
                               gain_next=parts["norm2"].weight, h=h)
         parts["feed_forward"].forward_add(ctx, h, ys[0])
-        norm2b = parts["norm2b"]
-        kernels.rms_post_norm([(ys[0], None)], x, norm2b.weight, n, norm2b.eps, norm2b.offset, self.mult)
+        ctx.pending_update = PendingSandwich([(ys[0], None)], x, parts["norm2b"], self.mult, n)
+
+
+class PendingSandwich:
+    """A sublayer's output that is still to be normed and added to the residual: x += mult * norm(y).  Whoever
+    reads x next makes the addition: a layer of the same kind together with its first norm (run(gain, h) also
+    leaves h = norm_next(x)), anyone else through flush_update."""
+
+    def __init__(self, joins, x: torch.Tensor, norm: Part, mult: float, n_rows: int) -> None:
+        self.joins, self.x, self.norm, self.mult, self.n_rows = joins, x, norm, mult, n_rows
+
+    def goes_with(self, norm_next: Part, x: torch.Tensor, n_rows: int) -> bool:
+        return (x is self.x and n_rows == self.n_rows and norm_next.eps == self.norm.eps
+                and norm_next.offset == self.norm.offset)
+
+    def run(self, gain_next: Optional[torch.Tensor], h: Optional[torch.Tensor]) -> None:
+        kernels.rms_post_norm(self.joins, self.x, self.norm.weight, self.n_rows, self.norm.eps, self.norm.offset,
+                              self.mult, gain_next=gain_next, h=h)
+
+
+def flush_update(ctx: StepContext) -> None:
+    """Makes the addition to the residual that a layer has left pending, if any."""
+    if ctx.pending_update is not None:
+        left, ctx.pending_update = ctx.pending_update, None
+        left.run(None, None)

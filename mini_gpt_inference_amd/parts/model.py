@@ -369,6 +369,7 @@ class DecoderModel:
         x = ws.get("residual", n, streams * self.spec.width, torch.float32)
         ctx.pending = None
         ctx.pending_streams = None
+        ctx.pending_update = None
         self.embedding.forward(ctx, self.position, x)
         if self.embedding_norm is not None:
             residual.settle(ctx, x, n)
@@ -377,9 +378,12 @@ class DecoderModel:
             layer = self.layers[run.layer]
             if not getattr(layer.arrangement, "takes_pending_streams", False):
                 _block.flush_streams(ctx, x, streams)
+            if not getattr(layer.arrangement, "takes_pending_update", False):
+                _block.flush_update(ctx)
             if not layer.arrangement.takes_pending_residual:
                 residual.settle(ctx, x, n)
             layer.arrangement.run(ctx, x, layer.parts, bindings, self.position)
+        _block.flush_update(ctx)
         m = ctx.m_rows
         # rows start 16 bytes apart at least: the sampling kernel then reads them four floats at a time
         # whatever the vocabulary's size (50257 is odd)
