@@ -164,15 +164,14 @@ extern "C" int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, i
 //   P[i][j] = (q_i . k_j) L^(i-j) for j <= i, else 0
 //   o_i     = sum_j P[i][j] v_j + L^(i+1) S^T q_i
 //   S      <- L^n S + sum_j L^(n-1-j) k_j v_j^T
-// A workgroup owns (request, head, 32 value channels): the columns of S are independent of each
+// A workgroup owns (request, head, 32 or 16 value channels): the columns of S are independent of each
 // other, so a head's value channels are dealt out over workgroups, each of which makes P for itself.
 // Queries and keys come ready (activation, rotation, scale) as float32 from state_inputs_kernel.
 
 #define DC_C 32        // tokens a chunk
-#define DC_EB 32       // value channels a workgroup
 #define DC_DMAX 128    // largest head size of this path
 #define DC_LDQ (DC_DMAX + 4)
-#define DC_LDE (DC_EB + 4)
+#define DC_LDP (DC_C + 4)
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
@@ -213,13 +212,15 @@ __global__ __launch_bounds__(256) void state_inputs_kernel(const void* __restric
   }
 }
 
+template <int EB>     // value channels a workgroup: 32, or 16 where that is what fills the machine
 __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     const float* __restrict__ qk, const void* __restrict__ z, int dtype, long ldz, int v_off, int n_head, int D, int E,
     int act, const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q, float* __restrict__ out, long ldo) {
-  __shared__ float Qs[DC_C][DC_LDQ], Ks[DC_C][DC_LDQ], Ss[DC_DMAX][DC_LDE], Vs[DC_C][DC_LDE], Ps[DC_C][DC_LDE];
+  constexpr int NJ = EB / 16;     // column tiles of the workgroup's value channels
+  __shared__ float Qs[DC_C][DC_LDQ], Ks[DC_C][DC_LDQ], Ss[DC_DMAX][EB + 4], Vs[DC_C][EB + 4], Ps[DC_C][DC_LDP];
   __shared__ float pw[DC_C + 1];
-  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * DC_EB, tid = threadIdx.x;
+  const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * EB, tid = threadIdx.x;
   const int slot = state_slots[r];
   const int t_begin = cu_q[r], t_end = cu_q[r + 1];
   if (slot < 0 || t_end <= t_begin) return;     // a request of the padding
@@ -231,15 +232,15 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
   if (tid <= DC_C) pw[tid] = tid == 0 ? 1.0f : expf((float)tid * log_l);
   float* st = state + ((long)slot * n_head + h) * (long)D * E;
   const bool fresh = positions[t_begin] == 0;
-  for (int i = tid; i < Dp * DC_EB; i += 256) {
-    const int d = i / DC_EB, c = i - d * DC_EB;
+  for (int i = tid; i < Dp * EB; i += 256) {
+    const int d = i / EB, c = i - d * EB;
     Ss[d][c] = (!fresh && d < D && e0 + c < E) ? st[(long)d * E + e0 + c] : 0.f;
   }
   const int ti = wave >> 1, tj = wave & 1;      // this wave's 16 x 16 tile of P and of the chunk's outputs
 
   // A chunk's rows travel from memory into registers while the chunk before is multiplied: thread tid holds
   // elements tid, tid + 256, ... of the chunk's [32, Dp] queries and keys and of its [32, 32] values.
-  constexpr int QK_PT = DC_C * DC_DMAX / 256, V_PT = DC_C * DC_EB / 256;
+  constexpr int QK_PT = DC_C * DC_DMAX / 256, V_PT = DC_C * EB / 256;
   float q_r[QK_PT], k_r[QK_PT], v_r[V_PT];
   auto fetch = [&](int t0) {
     const int nt = t_end - t0 < DC_C ? t_end - t0 : DC_C;      // may be <= 0
@@ -253,7 +254,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     }
 #pragma unroll
     for (int u = 0; u < V_PT; ++u) {
-      const int i = tid + u * 256, tt = i / DC_EB, c = i - tt * DC_EB;
+      const int i = tid + u * 256, tt = i / EB, c = i - tt * EB;
       v_r[u] = (tt < nt && e0 + c < E)
                    ? ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + e0 + c), act) : 0.f;
     }
@@ -274,7 +275,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
 #pragma unroll
     for (int u = 0; u < V_PT; ++u) {
       const int i = tid + u * 256;
-      Vs[i / DC_EB][i % DC_EB] = v_r[u];
+      Vs[i / EB][i % EB] = v_r[u];
     }
     __syncthreads();
     fetch(t0 + DC_C);     // (behind the last chunk: no token is left, nothing is loaded)
@@ -293,40 +294,42 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
       }
     }
     __syncthreads();
-    // ---- o = P V + L^(i+1) Q S
-    {
+    // ---- o = P V + L^(i+1) Q S: the tiles (oi, oj) of the chunk's [32, EB] outputs
+    for (int t = wave; t < 2 * NJ; t += 4) {
+      const int oi = t / NJ, oj = t - oi * NJ;
       f32x4_t a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
-      for (int k0 = 0; k0 < (ti + 1) * 16; k0 += 4)
-        a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[ti * 16 + r16][k0 + g], Vs[k0 + g][tj * 16 + r16], a1, 0, 0, 0);
+      for (int k0 = 0; k0 < (oi + 1) * 16; k0 += 4)
+        a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[oi * 16 + r16][k0 + g], Vs[k0 + g][oj * 16 + r16], a1, 0, 0, 0);
 #pragma unroll 4
       for (int k0 = 0; k0 < Dp; k0 += 4)
-        a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ss[k0 + g][tj * 16 + r16], a2, 0, 0, 0);
+        a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[oi * 16 + r16][k0 + g], Ss[k0 + g][oj * 16 + r16], a2, 0, 0, 0);
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
-        const int i = ti * 16 + 4 * g + v, c = e0 + tj * 16 + r16;
+        const int i = oi * 16 + 4 * g + v, c = e0 + oj * 16 + r16;
         if (i < nt && c < E) out[(long)(t0 + i) * ldo + (long)h * E + c] = a1[v] + pw[i + 1] * a2[v];
       }
     }
     __syncthreads();     // every wave has read the old S
-    // ---- S <- L^n S + sum_t L^(n-1-t) k_t v_t^T: the tiles (di, tj) with di = ti, ti + 2, ...
-    for (int di = ti; di * 16 < Dp; di += 2) {
+    // ---- S <- L^n S + sum_t L^(n-1-t) k_t v_t^T: the tiles (di, sj) of the [Dp, EB] state, dealt out over the waves
+    for (int t = wave; t < (Dp >> 4) * NJ; t += 4) {
+      const int di = t / NJ, sj = t - di * NJ;
       f32x4_t acc;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[v] = pw[nt] * Ss[di * 16 + 4 * g + v][tj * 16 + r16];
+      for (int v = 0; v < 4; ++v) acc[v] = pw[nt] * Ss[di * 16 + 4 * g + v][sj * 16 + r16];
 #pragma unroll
       for (int k0 = 0; k0 < DC_C; k0 += 4) {
-        const int t = k0 + g;
-        const float w = t < nt ? pw[nt - 1 - t] : 0.f;
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[t][di * 16 + r16] * w, Vs[t][tj * 16 + r16], acc, 0, 0, 0);
+        const int tk = k0 + g;
+        const float w = tk < nt ? pw[nt - 1 - tk] : 0.f;
+        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[tk][di * 16 + r16] * w, Vs[tk][sj * 16 + r16], acc, 0, 0, 0);
       }
 #pragma unroll
-      for (int v = 0; v < 4; ++v) Ss[di * 16 + 4 * g + v][tj * 16 + r16] = acc[v];
+      for (int v = 0; v < 4; ++v) Ss[di * 16 + 4 * g + v][sj * 16 + r16] = acc[v];
     }
   }
   __syncthreads();
-  for (int i = tid; i < D * DC_EB; i += 256) {
-    const int d = i / DC_EB, c = i - d * DC_EB;
+  for (int i = tid; i < D * EB; i += 256) {
+    const int d = i / EB, c = i - d * EB;
     if (e0 + c < E) st[(long)d * E + e0 + c] = Ss[d][c];
   }
 }
@@ -349,7 +352,12 @@ extern "C" int mgpt_decay_state_chunked(const void* z, int dtype, long ldz, int 
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
   hipLaunchKernelGGL(state_inputs_kernel, dim3(n_tokens), dim3(256), 0, stream, z, dtype, ldz, q_off, k_off, n_head, D, act,
                      positions, rot_dims ? freq : nullptr, rot_dims, k_scale, qk, n_tokens);
-  hipLaunchKernelGGL(decay_state_chunk_kernel, dim3(n_req, n_head, (E + DC_EB - 1) / DC_EB), dim3(256), 0, stream, qk, z,
-                     dtype, ldz, v_off, n_head, D, E, act, positions, decay, state, state_slots, cu_q, out, ldo);
+  // 32 value channels a workgroup; 16 where that many workgroups would leave compute units idle
+  if ((long)n_req * n_head * ((E + 31) / 32) >= 256)
+    hipLaunchKernelGGL(decay_state_chunk_kernel<32>, dim3(n_req, n_head, (E + 31) / 32), dim3(256), 0, stream, qk, z, dtype,
+                       ldz, v_off, n_head, D, E, act, positions, decay, state, state_slots, cu_q, out, ldo);
+  else
+    hipLaunchKernelGGL(decay_state_chunk_kernel<16>, dim3(n_req, n_head, (E + 15) / 16), dim3(256), 0, stream, qk, z, dtype,
+                       ldz, v_off, n_head, D, E, act, positions, decay, state, state_slots, cu_q, out, ldo);
   return mgpt_last_error();
 }

@@ -152,6 +152,49 @@ __global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int 
     store_f(h, h_dtype, base + c, x[base + c] * rx * (offset + gain_next[c]));
 }
 
+// The same step for one branch and rows of up to 256 * PT values: every value is loaded once (the row, the
+// sublayer's output and both gains are in registers before the first sum), one trip to memory instead of three.
+template <int PT>
+__global__ __launch_bounds__(256) void rms_post_norm_row_kernel(float* __restrict__ y, float* __restrict__ x,
+                                                                const float* __restrict__ gain_post, float offset, float eps,
+                                                                float mult, const float* __restrict__ gain_next,
+                                                                void* __restrict__ h, int h_dtype, int n_rows, int width) {
+  __shared__ float scratch[4];
+  const long base = (long)blockIdx.x * width;
+  float yv[PT], xv[PT], gp[PT], gn[PT];
+#pragma unroll
+  for (int u = 0; u < PT; ++u) {
+    const int c = threadIdx.x + u * 256;
+    const bool ok = c < width;
+    yv[u] = ok ? y[base + c] : 0.f;
+    xv[u] = ok ? x[base + c] : 0.f;
+    gp[u] = ok ? gain_post[c] : 0.f;
+    gn[u] = (ok && gain_next) ? gain_next[c] : 0.f;
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int u = 0; u < PT; ++u) ss = fmaf(yv[u], yv[u], ss);
+  const float ry = mult / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+  float sx = 0.f;
+#pragma unroll
+  for (int u = 0; u < PT; ++u) {
+    const int c = threadIdx.x + u * 256;
+    xv[u] = xv[u] + yv[u] * ry * (offset + gp[u]);
+    if (c < width) {
+      x[base + c] = xv[u];
+      y[base + c] = 0.f;
+      sx = fmaf(xv[u], xv[u], sx);
+    }
+  }
+  if (!gain_next) return;
+  const float rx = 1.0f / sqrtf(block_sum_256(sx, scratch) / (float)width + eps);
+#pragma unroll
+  for (int u = 0; u < PT; ++u) {
+    const int c = threadIdx.x + u * 256;
+    if (c < width) store_f(h, h_dtype, base + c, xv[u] * rx * (offset + gn[u]));
+  }
+}
+
 // y_ptrs / gain_ptrs: n_branches device pointers each (float32 [n_rows, width] buffers; [width] gains, unused
 // with one branch).  x, y: contiguous float32 rows.
 extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, const float* g0, const float* g1,
@@ -165,7 +208,15 @@ extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, co
   RmsBranches br = {{y0, y1, y2, y3}, {g0, g1, g2, g3}};
   for (int b = 0; b < n_branches; ++b)
     if (!br.y[b] || (n_branches > 1 && !br.gain[b])) return MGPT_ERR_NULL;
-  hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, x, gain_post,
-                     offset, eps, mult, gain_next, h, h_dtype, n_rows, width);
+#define RPN_ROW(PT)                                                                                                  \
+  hipLaunchKernelGGL(rms_post_norm_row_kernel<PT>, dim3(n_rows), dim3(256), 0, stream, y0, x, gain_post, offset, eps, mult, \
+                     gain_next, h, h_dtype, n_rows, width)
+  if (n_branches == 1 && width <= 256 * 4) RPN_ROW(4);
+  else if (n_branches == 1 && width <= 256 * 8) RPN_ROW(8);
+  else if (n_branches == 1 && width <= 256 * 16) RPN_ROW(16);
+  else
+    hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, x, gain_post,
+                       offset, eps, mult, gain_next, h, h_dtype, n_rows, width);
+#undef RPN_ROW
   return mgpt_last_error();
 }

@@ -80,7 +80,8 @@ def test_rms_norm_segments_gate_and_accumulate(dtype, groups, width, stride):
 
 
 @pytest.mark.parametrize("h_dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("branches,n,width", [(1, 3, 40), (2, 70, 64), (3, 5, 300), (4, 2, 1030), (1, 9, 2048)])
+@pytest.mark.parametrize("branches,n,width", [(1, 3, 40), (2, 70, 64), (3, 5, 300), (4, 2, 1030), (1, 9, 2048), (1, 5, 3000),
+                                              (1, 2, 5000), (1, 4, 1024)])
 def test_the_step_between_two_sublayers(h_dtype, branches, n, width):
     g = torch.Generator().manual_seed(branches + width)
     x = _rnd(g, n + 1, width, scale=3.0)
@@ -236,7 +237,7 @@ def test_decaying_state_whole_in_portions_and_slots_used_again(dtype, H, D, E):
     lens = [37, 1, 12]
     z, k_off, v_off, g_off = _state_case(g, dtype, lens, H, D, E)
     n = sum(lens)
-    decay = torch.tensor([0.999, 0.6, 0.9][:H])
+    decay = torch.tensor(([0.999, 0.6, 0.9] * 3)[:H])
     dims = D - D % 2 if D >= 2 else 0
     freq = _freq(dims, 1000.0) if dims else None
     for variant in ("retention", "lightning"):
@@ -300,7 +301,7 @@ def test_decaying_state_whole_in_portions_and_slots_used_again(dtype, H, D, E):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("H,D,E", [(2, 16, 24), (1, 64, 64), (2, 128, 128), (3, 20, 12), (1, 128, 200), (2, 8, 256),
-                                   (1, 1, 1), (1, 30, 33)])
+                                   (1, 1, 1), (1, 30, 33), (8, 16, 200), (9, 64, 160)])     # (the last two: 32 channels a workgroup)
 def test_decaying_state_a_chunk_at_a_time(dtype, H, D, E):
     """The matrix-core form for prompt portions against the plain recurrence: requests whose lengths are
     below, at and beyond the chunk of 32 tokens, in one step; then cut into portions that end inside
@@ -309,7 +310,7 @@ def test_decaying_state_a_chunk_at_a_time(dtype, H, D, E):
     lens = [70, 1, 32, 33]
     n = sum(lens)
     z, k_off, v_off, g_off = _state_case(g, dtype, lens, H, D, E)
-    decay = torch.tensor([0.999, 0.6, 0.9][:H])
+    decay = torch.tensor(([0.999, 0.6, 0.9] * 3)[:H])
     dims = D - D % 2 if D >= 2 else 0
     for variant in ("rotated", "silu"):
         f = P.silu if variant == "silu" else (lambda t: t)
