@@ -14,7 +14,8 @@
 // One workgroup per (request, head) walks the request's tokens of this step in order, whatever
 // their number (a prompt, a portion of one, one decoded token), from the state that the step
 // before left in the request's slot, and leaves the new state there.  The state lives in
-// registers: thread (dg, e) owns S[d][e] for d = dg, dg + NG, ...; the tokens' q, k, v are staged
+// registers: thread (dg, e) owns S[d][e] for d = dg, dg + NG, ... (256 threads a workgroup, or 1,024 for a
+// large state, so that a thread's share stays small); the tokens' q, k, v are staged
 // through LDS eight at a time, and the partial sums over dg meet there once per eight tokens.
 #include "common.h"
 #include "dtype_io.h"
@@ -25,18 +26,18 @@
 
 __device__ __forceinline__ float ds_act(float v, int act) { return act == 1 ? v / (1.0f + expf(-v)) : v; }
 
-template <int R>
-__global__ __launch_bounds__(256) void decay_state_kernel(
+template <int R, int NT>     // state values a thread, threads a workgroup
+__global__ __launch_bounds__(NT) void decay_state_kernel(
     const void* __restrict__ z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head, int D, int E,
     int act, const int* __restrict__ positions, const float* __restrict__ freq, int rot_dims, float k_scale,
     const float* __restrict__ decay, float* __restrict__ state, const int* __restrict__ state_slots,
     const int* __restrict__ cu_q, float norm_eps, void* __restrict__ out, int out_dtype, long ldo) {
-  __shared__ float q_s[DS_TC][DS_MAX], k_s[DS_TC][DS_MAX], v_s[DS_TC][DS_MAX], red[DS_TC][256];
+  __shared__ float q_s[DS_TC][DS_MAX], k_s[DS_TC][DS_MAX], v_s[DS_TC][DS_MAX], red[DS_TC][NT];
   const int r = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int slot = state_slots[r];
   const int t_begin = cu_q[r], t_end = cu_q[r + 1];
   if (slot < 0 || t_end <= t_begin) return;     // a request of the padding
-  const int NG = 256 / E < D ? 256 / E : D;     // groups of threads over d (at least 1: E <= 256)
+  const int NG = NT / E < D ? NT / E : D;       // groups of threads over d (at least 1: E <= 256)
   const bool owner = tid < NG * E;
   const int e = tid % E, dg = tid / E;
   const int count = owner ? (D - dg + NG - 1) / NG : 0;
@@ -52,19 +53,19 @@ __global__ __launch_bounds__(256) void decay_state_kernel(
   for (int t0 = t_begin; t0 < t_end; t0 += DS_TC) {
     const int nt = t_end - t0 < DS_TC ? t_end - t0 : DS_TC;
     __syncthreads();     // the chunk before is read
-    for (int i = tid; i < nt * D; i += 256) {
+    for (int i = tid; i < nt * D; i += NT) {
       const int tt = i / D, d = i - tt * D;
       const long row = (long)(t0 + tt) * ldz + (long)h * D + d;
       q_s[tt][d] = ds_act(load_f(z, dtype, row + q_off), act);
       k_s[tt][d] = ds_act(load_f(z, dtype, row + k_off), act);
     }
-    for (int i = tid; i < nt * E; i += 256) {
+    for (int i = tid; i < nt * E; i += NT) {
       const int tt = i / E, c = i - tt * E;
       v_s[tt][c] = ds_act(load_f(z, dtype, (long)(t0 + tt) * ldz + v_off + (long)h * E + c), act);
     }
     __syncthreads();
     if (freq) {
-      for (int i = tid; i < nt * half; i += 256) {
+      for (int i = tid; i < nt * half; i += NT) {
         const int tt = i / half, c = i - tt * half;
         const float a = (float)positions[t0 + tt] * freq[c];
         const float co = cosf(a), si = sinf(a);
@@ -75,12 +76,12 @@ __global__ __launch_bounds__(256) void decay_state_kernel(
         k_s[tt][c + half] = (kw * co + ku * si) * k_scale;
       }
       if (k_scale != 1.0f)
-        for (int i = tid; i < nt * (D - rot_dims); i += 256) {
+        for (int i = tid; i < nt * (D - rot_dims); i += NT) {
           const int tt = i / (D - rot_dims), c = rot_dims + i - tt * (D - rot_dims);
           k_s[tt][c] *= k_scale;
         }
     } else if (k_scale != 1.0f) {
-      for (int i = tid; i < nt * D; i += 256) k_s[i / D][i % D] *= k_scale;
+      for (int i = tid; i < nt * D; i += NT) k_s[i / D][i % D] *= k_scale;
     }
     __syncthreads();
     if (owner) {
@@ -100,7 +101,7 @@ __global__ __launch_bounds__(256) void decay_state_kernel(
     }
     __syncthreads();
     // a wave a token: the sums over dg in order, the head's norm, the gate, the store
-    for (int tt = wave; tt < nt; tt += 4) {
+    for (int tt = wave; tt < nt; tt += NT / 64) {
       float ss = 0.f;
       for (int c = lane; c < E; c += 64) {
         float o = 0.f;
@@ -141,18 +142,22 @@ extern "C" int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, i
       rot_dims > D || (act != 0 && act != 1))
     return MGPT_ERR_BAD_SHAPE;
   if (n_head > 65535) return MGPT_ERR_TOO_LARGE;
-  const int ng = 256 / E < D ? 256 / E : D;
-  const int per_thread = (D + ng - 1) / ng;
-  dim3 grid(n_req, n_head), block(256);
-#define DS_LAUNCH(R)                                                                                                   \
-  hipLaunchKernelGGL(decay_state_kernel<R>, grid, block, 0, stream, z, dtype, ldz, q_off, k_off, v_off, g_off, n_head, D, E, \
-                     act, positions, rot_dims ? freq : nullptr, rot_dims, k_scale, decay, state, state_slots, cu_q, norm_eps, \
-                     out, out_dtype, ldo)
-  if (per_thread <= 8) DS_LAUNCH(8);
-  else if (per_thread <= 32) DS_LAUNCH(32);
-  else if (per_thread <= 64) DS_LAUNCH(64);
-  else if (per_thread <= 128) DS_LAUNCH(128);
-  else return MGPT_ERR_BAD_SHAPE;     // a state of more than 128 values a thread
+  // a workgroup of 256 threads while a thread then owns at most 16 values of the state, else one of 1,024
+  auto per_thread = [&](int threads) {
+    const int ng = threads / E < D ? threads / E : D;
+    return (D + ng - 1) / ng;
+  };
+  dim3 grid(n_req, n_head);
+#define DS_LAUNCH(R, NT)                                                                                                   \
+  hipLaunchKernelGGL((decay_state_kernel<R, NT>), grid, dim3(NT), 0, stream, z, dtype, ldz, q_off, k_off, v_off, g_off, n_head, \
+                     D, E, act, positions, rot_dims ? freq : nullptr, rot_dims, k_scale, decay, state, state_slots, cu_q,   \
+                     norm_eps, out, out_dtype, ldo)
+  if (per_thread(256) <= 8) DS_LAUNCH(8, 256);
+  else if (per_thread(256) <= 16) DS_LAUNCH(16, 256);
+  else if (per_thread(1024) <= 16) DS_LAUNCH(16, 1024);
+  else if (per_thread(1024) <= 32) DS_LAUNCH(32, 1024);
+  else if (per_thread(1024) <= 64) DS_LAUNCH(64, 1024);
+  else return MGPT_ERR_BAD_SHAPE;
 #undef DS_LAUNCH
   return mgpt_last_error();
 }

@@ -152,37 +152,61 @@ __global__ __launch_bounds__(256) void rms_post_norm_kernel(RmsBranches br, int 
     store_f(h, h_dtype, base + c, x[base + c] * rx * (offset + gain_next[c]));
 }
 
-// The same step for one branch and rows of up to 256 * PT values: every value is loaded once (the row, the
-// sublayer's output and both gains are in registers before the first sum), one trip to memory instead of three.
-template <int PT>
-__global__ __launch_bounds__(256) void rms_post_norm_row_kernel(float* __restrict__ y, float* __restrict__ x,
+// The same step for one or two branches and rows of up to 256 * PT values: every value is loaded once (the row,
+// the sublayers' outputs and all gains are in registers before the first sum), one trip to memory instead of
+// three or five.
+template <int PT, int NB>
+__global__ __launch_bounds__(256) void rms_post_norm_row_kernel(RmsBranches br, float coef, float* __restrict__ x,
                                                                 const float* __restrict__ gain_post, float offset, float eps,
                                                                 float mult, const float* __restrict__ gain_next,
                                                                 void* __restrict__ h, int h_dtype, int n_rows, int width) {
   __shared__ float scratch[4];
   const long base = (long)blockIdx.x * width;
-  float yv[PT], xv[PT], gp[PT], gn[PT];
+  float yv[NB][PT], jg[NB][PT], xv[PT], gp[PT], gn[PT];
 #pragma unroll
   for (int u = 0; u < PT; ++u) {
     const int c = threadIdx.x + u * 256;
     const bool ok = c < width;
-    yv[u] = ok ? y[base + c] : 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      yv[b][u] = ok ? br.y[b][base + c] : 0.f;
+      jg[b][u] = (ok && NB > 1) ? br.gain[b][c] : 1.f;
+    }
     xv[u] = ok ? x[base + c] : 0.f;
     gp[u] = ok ? gain_post[c] : 0.f;
     gn[u] = (ok && gain_next) ? gain_next[c] : 0.f;
   }
+  if (NB > 1) {
+    // the branches' outputs, each normed with its own plain gain, averaged
+    float r[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      float ss = 0.f;
+#pragma unroll
+      for (int u = 0; u < PT; ++u) ss = fmaf(yv[b][u], yv[b][u], ss);
+      r[b] = coef / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
+    }
+#pragma unroll
+    for (int u = 0; u < PT; ++u) {
+      float v = 0.f;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) v = fmaf(yv[b][u] * r[b], jg[b][u], v);
+      yv[0][u] = v;
+    }
+  }
   float ss = 0.f;
 #pragma unroll
-  for (int u = 0; u < PT; ++u) ss = fmaf(yv[u], yv[u], ss);
+  for (int u = 0; u < PT; ++u) ss = fmaf(yv[0][u], yv[0][u], ss);
   const float ry = mult / sqrtf(block_sum_256(ss, scratch) / (float)width + eps);
   float sx = 0.f;
 #pragma unroll
   for (int u = 0; u < PT; ++u) {
     const int c = threadIdx.x + u * 256;
-    xv[u] = xv[u] + yv[u] * ry * (offset + gp[u]);
+    xv[u] = xv[u] + yv[0][u] * ry * (offset + gp[u]);
     if (c < width) {
       x[base + c] = xv[u];
-      y[base + c] = 0.f;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) br.y[b][base + c] = 0.f;
       sx = fmaf(xv[u], xv[u], sx);
     }
   }
@@ -208,12 +232,14 @@ extern "C" int mgpt_rms_post_norm(float* y0, float* y1, float* y2, float* y3, co
   RmsBranches br = {{y0, y1, y2, y3}, {g0, g1, g2, g3}};
   for (int b = 0; b < n_branches; ++b)
     if (!br.y[b] || (n_branches > 1 && !br.gain[b])) return MGPT_ERR_NULL;
-#define RPN_ROW(PT)                                                                                                  \
-  hipLaunchKernelGGL(rms_post_norm_row_kernel<PT>, dim3(n_rows), dim3(256), 0, stream, y0, x, gain_post, offset, eps, mult, \
-                     gain_next, h, h_dtype, n_rows, width)
-  if (n_branches == 1 && width <= 256 * 4) RPN_ROW(4);
-  else if (n_branches == 1 && width <= 256 * 8) RPN_ROW(8);
-  else if (n_branches == 1 && width <= 256 * 16) RPN_ROW(16);
+#define RPN_ROW(PT, NB)                                                                                              \
+  hipLaunchKernelGGL((rms_post_norm_row_kernel<PT, NB>), dim3(n_rows), dim3(256), 0, stream, br, coef, x, gain_post, offset, \
+                     eps, mult, gain_next, h, h_dtype, n_rows, width)
+  if (n_branches == 1 && width <= 256 * 4) RPN_ROW(4, 1);
+  else if (n_branches == 1 && width <= 256 * 8) RPN_ROW(8, 1);
+  else if (n_branches == 1 && width <= 256 * 16) RPN_ROW(16, 1);
+  else if (n_branches == 2 && width <= 256 * 4) RPN_ROW(4, 2);
+  else if (n_branches == 2 && width <= 256 * 8) RPN_ROW(8, 2);
   else
     hipLaunchKernelGGL(rms_post_norm_kernel, dim3(n_rows), dim3(256), 0, stream, br, n_branches, coef, x, gain_post,
                        offset, eps, mult, gain_next, h, h_dtype, n_rows, width);

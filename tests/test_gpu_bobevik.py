@@ -81,7 +81,7 @@ def test_rms_norm_segments_gate_and_accumulate(dtype, groups, width, stride):
 
 @pytest.mark.parametrize("h_dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("branches,n,width", [(1, 3, 40), (2, 70, 64), (3, 5, 300), (4, 2, 1030), (1, 9, 2048), (1, 5, 3000),
-                                              (1, 2, 5000), (1, 4, 1024)])
+                                              (1, 2, 5000), (1, 4, 1024), (2, 3, 2048), (2, 2, 2100)])
 def test_the_step_between_two_sublayers(h_dtype, branches, n, width):
     g = torch.Generator().manual_seed(branches + width)
     x = _rnd(g, n + 1, width, scale=3.0)
