@@ -41,9 +41,12 @@ __device__ __forceinline__ float block_sum(float v, float* scratch) {
   return blockDim.x == 128 ? scratch[0] + scratch[1] : (scratch[0] + scratch[1]) + (scratch[2] + scratch[3]);
 }
 
-// one workgroup per segment: a wave for a narrow one (a head), four for a wide one (a row of the model's width)
+// one workgroup per segment: a wave for a narrow one (a head), four for a wide one (a row of the model's width).
+// PT > 0: a thread keeps its PT values of the segment in registers between the two passes (segments of up to
+// PT * threads values); PT = 0: the second pass reads them again.
+template <int PT>
 __global__ __launch_bounds__(256) void rms_norm_kernel(
-    const void* __restrict__ x, int x_dtype, long ldx, const int* __restrict__ rows,
+    const void* x, int x_dtype, long ldx, const int* __restrict__ rows,      // (out may be x: the norm in place)
     const float* __restrict__ gain, float offset, float eps, float mult, const void* __restrict__ gate,
     int gate_dtype, long ldg, int gate_act, void* out, int out_dtype, long ldo, int accumulate,
     float* __restrict__ zero, long ldz, int zero_width, int n_rows, int groups, int x_gstride, int o_gstride,
@@ -54,21 +57,41 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   const int src = rows ? rows[row] : row;
   const long xb = (long)src * ldx + (long)g * x_gstride;
   const int step = blockDim.x;
+  float xv[PT > 0 ? PT : 1];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < width; c += step) {
-    const float v = load_f(x, x_dtype, xb + c);
-    ss = fmaf(v, v, ss);
+  if (PT > 0) {
+#pragma unroll
+    for (int u = 0; u < PT; ++u) {
+      const int c = threadIdx.x + u * step;
+      xv[u] = c < width ? load_f(x, x_dtype, xb + c) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < PT; ++u) ss = fmaf(xv[u], xv[u], ss);
+  } else {
+    for (int c = threadIdx.x; c < width; c += step) {
+      const float v = load_f(x, x_dtype, xb + c);
+      ss = fmaf(v, v, ss);
+    }
   }
   ss = block_sum(ss, scratch);
   const float r = mult / sqrtf(ss / (float)width + eps);
   const long ob = (long)row * ldo + (long)g * o_gstride;
   const long gb = (long)row * ldg + (long)g * o_gstride;
-  for (int c = threadIdx.x; c < width; c += step) {
-    float v = load_f(x, x_dtype, xb + c) * r;
+  auto finish = [&](int c, float v) {
+    v *= r;
     if (gain) v *= offset + gain[(long)g * width + c];
     if (gate) v *= rms_gate_act(load_f(gate, gate_dtype, gb + c), gate_act);
     if (accumulate) v += load_f(out, out_dtype, ob + c);
     store_f(out, out_dtype, ob + c, v);
+  };
+  if (PT > 0) {
+#pragma unroll
+    for (int u = 0; u < PT; ++u) {
+      const int c = threadIdx.x + u * step;
+      if (c < width) finish(c, xv[u]);
+    }
+  } else {
+    for (int c = threadIdx.x; c < width; c += step) finish(c, load_f(x, x_dtype, xb + c));
   }
   if (zero && g == 0)
     for (int c = threadIdx.x; c < zero_width; c += step) zero[(long)row * ldz + c] = 0.f;
@@ -86,9 +109,15 @@ extern "C" int mgpt_rms_norm(const void* x, int x_dtype, long ldx, const int* ro
   const long segs = (long)n_rows * groups;
   if (segs > 0x7fffffffL) return MGPT_ERR_TOO_LARGE;
   const int threads = width <= 256 ? 64 : (width <= 512 ? 128 : 256);
-  hipLaunchKernelGGL(rms_norm_kernel, dim3((unsigned)segs), dim3(threads), 0, stream, x, x_dtype, ldx, rows,
-                     gain, offset, eps, mult, gate, gate_dtype, ldg, gate_act, out, out_dtype, ldo, accumulate, zero,
-                     ldz, zero_width, n_rows, groups, x_gstride, o_gstride, width);
+#define RN_LAUNCH(PT)                                                                                              \
+  hipLaunchKernelGGL(rms_norm_kernel<PT>, dim3((unsigned)segs), dim3(threads), 0, stream, x, x_dtype, ldx, rows, gain,  \
+                     offset, eps, mult, gate, gate_dtype, ldg, gate_act, out, out_dtype, ldo, accumulate, zero, ldz,   \
+                     zero_width, n_rows, groups, x_gstride, o_gstride, width)
+  const int per_thread = (width + threads - 1) / threads;
+  if (per_thread <= 4) RN_LAUNCH(4);
+  else if (per_thread <= 16) RN_LAUNCH(16);
+  else RN_LAUNCH(0);
+#undef RN_LAUNCH
   return mgpt_last_error();
 }
 

@@ -34,7 +34,7 @@ def _d(t):
 
 # ---------------------------------------------------------------- kernels, one at a time
 @pytest.mark.parametrize("out_dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("n,width", [(1, 8), (5, 40), (70, 256), (3, 1000), (2, 4100)])
+@pytest.mark.parametrize("n,width", [(1, 8), (5, 40), (70, 256), (3, 1000), (2, 4100), (4, 2048), (2, 300)])
 def test_rms_norm_rows(out_dtype, n, width):
     g = torch.Generator().manual_seed(width)
     x = _rnd(g, n + 1, width, scale=3.0)
