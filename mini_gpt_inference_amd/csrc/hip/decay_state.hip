@@ -223,7 +223,12 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     int act, const int* __restrict__ positions, const float* __restrict__ decay, float* __restrict__ state,
     const int* __restrict__ state_slots, const int* __restrict__ cu_q, float* __restrict__ out, long ldo) {
   constexpr int NJ = EB / 16;     // column tiles of the workgroup's value channels
-  __shared__ float Qs[DC_C][DC_LDQ], Ks[DC_C][DC_LDQ], Ss[DC_DMAX][EB + 4], Vs[DC_C][EB + 4], Ps[DC_C][DC_LDP];
+  // queries and keys [token][d]; the state and the values transposed, [value channel][d] and [value channel][token];
+  // P [token][token].  Every product's index of summation runs along a row, so that a lane's operands of four
+  // matrix instructions are one 16-byte read: instruction s of such a group takes k = k0 + 4 g + s from lane (r16, g)
+  // (any dealing of a stretch's 16 values of k over four instructions gives the same sum, if both operands agree).
+  __shared__ __attribute__((aligned(16))) float Qs[DC_C][DC_LDQ], Ks[DC_C][DC_LDQ], St[EB][DC_LDQ], Vt[EB][DC_LDP],
+      Ps[DC_C][DC_LDP];
   __shared__ float pw[DC_C + 1];
   const int r = blockIdx.x, h = blockIdx.y, e0 = blockIdx.z * EB, tid = threadIdx.x;
   const int slot = state_slots[r];
@@ -239,7 +244,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
   const bool fresh = positions[t_begin] == 0;
   for (int i = tid; i < Dp * EB; i += 256) {
     const int d = i / EB, c = i - d * EB;
-    Ss[d][c] = (!fresh && d < D && e0 + c < E) ? st[(long)d * E + e0 + c] : 0.f;
+    St[c][d] = (!fresh && d < D && e0 + c < E) ? st[(long)d * E + e0 + c] : 0.f;
   }
   const int ti = wave >> 1, tj = wave & 1;      // this wave's 16 x 16 tile of P and of the chunk's outputs
 
@@ -280,7 +285,7 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
 #pragma unroll
     for (int u = 0; u < V_PT; ++u) {
       const int i = tid + u * 256;
-      Vs[i / EB][i % EB] = v_r[u];
+      Vt[i % EB][i / EB] = v_r[u];
     }
     __syncthreads();
     fetch(t0 + DC_C);     // (behind the last chunk: no token is left, nothing is loaded)
@@ -288,9 +293,13 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     {
       f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
       if (tj <= ti) {
-#pragma unroll 4
-        for (int k0 = 0; k0 < Dp; k0 += 4)
-          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[ti * 16 + r16][k0 + g], Ks[tj * 16 + r16][k0 + g], acc, 0, 0, 0);
+#pragma unroll 2
+        for (int k0 = 0; k0 < Dp; k0 += 16) {
+          const f32x4_t a = *reinterpret_cast<const f32x4_t*>(&Qs[ti * 16 + r16][k0 + 4 * g]);
+          const f32x4_t b = *reinterpret_cast<const f32x4_t*>(&Ks[tj * 16 + r16][k0 + 4 * g]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) acc = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], acc, 0, 0, 0);
+        }
       }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
@@ -303,12 +312,19 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     for (int t = wave; t < 2 * NJ; t += 4) {
       const int oi = t / NJ, oj = t - oi * NJ;
       f32x4_t a1 = {0.f, 0.f, 0.f, 0.f}, a2 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-      for (int k0 = 0; k0 < (oi + 1) * 16; k0 += 4)
-        a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(Ps[oi * 16 + r16][k0 + g], Vs[k0 + g][oj * 16 + r16], a1, 0, 0, 0);
-#pragma unroll 4
-      for (int k0 = 0; k0 < Dp; k0 += 4)
-        a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(Qs[oi * 16 + r16][k0 + g], Ss[k0 + g][oj * 16 + r16], a2, 0, 0, 0);
+      for (int k0 = 0; k0 < (oi + 1) * 16; k0 += 16) {
+        const f32x4_t a = *reinterpret_cast<const f32x4_t*>(&Ps[oi * 16 + r16][k0 + 4 * g]);
+        const f32x4_t b = *reinterpret_cast<const f32x4_t*>(&Vt[oj * 16 + r16][k0 + 4 * g]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a1 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], a1, 0, 0, 0);
+      }
+#pragma unroll 2
+      for (int k0 = 0; k0 < Dp; k0 += 16) {
+        const f32x4_t a = *reinterpret_cast<const f32x4_t*>(&Qs[oi * 16 + r16][k0 + 4 * g]);
+        const f32x4_t b = *reinterpret_cast<const f32x4_t*>(&St[oj * 16 + r16][k0 + 4 * g]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) a2 = __builtin_amdgcn_mfma_f32_16x16x4f32(a[e], b[e], a2, 0, 0, 0);
+      }
 #pragma unroll
       for (int v = 0; v < 4; ++v) {
         const int i = oi * 16 + 4 * g + v, c = e0 + oj * 16 + r16;
@@ -319,23 +335,27 @@ __global__ __launch_bounds__(256) void decay_state_chunk_kernel(
     // ---- S <- L^n S + sum_t L^(n-1-t) k_t v_t^T: the tiles (di, sj) of the [Dp, EB] state, dealt out over the waves
     for (int t = wave; t < (Dp >> 4) * NJ; t += 4) {
       const int di = t / NJ, sj = t - di * NJ;
-      f32x4_t acc;
+      f32x4_t* mine = reinterpret_cast<f32x4_t*>(&St[sj * 16 + r16][di * 16 + 4 * g]);     // rows d = 4 g + v of column r16
+      f32x4_t acc = *mine;
 #pragma unroll
-      for (int v = 0; v < 4; ++v) acc[v] = pw[nt] * Ss[di * 16 + 4 * g + v][sj * 16 + r16];
+      for (int v = 0; v < 4; ++v) acc[v] *= pw[nt];
 #pragma unroll
-      for (int k0 = 0; k0 < DC_C; k0 += 4) {
-        const int tk = k0 + g;
-        const float w = tk < nt ? pw[nt - 1 - tk] : 0.f;
-        acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[tk][di * 16 + r16] * w, Vs[tk][sj * 16 + r16], acc, 0, 0, 0);
+      for (int k0 = 0; k0 < DC_C; k0 += 16) {
+        const f32x4_t b = *reinterpret_cast<const f32x4_t*>(&Vt[sj * 16 + r16][k0 + 4 * g]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int tk = k0 + 4 * g + e;
+          const float w = tk < nt ? pw[nt - 1 - tk] : 0.f;
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(Ks[tk][di * 16 + r16] * w, b[e], acc, 0, 0, 0);
+        }
       }
-#pragma unroll
-      for (int v = 0; v < 4; ++v) Ss[di * 16 + 4 * g + v][sj * 16 + r16] = acc[v];
+      *mine = acc;
     }
   }
   __syncthreads();
   for (int i = tid; i < D * EB; i += 256) {
     const int d = i / EB, c = i - d * EB;
-    if (e0 + c < E) st[(long)d * E + e0 + c] = Ss[d][c];
+    if (e0 + c < E) st[(long)d * E + e0 + c] = St[c][d];
   }
 }
 
