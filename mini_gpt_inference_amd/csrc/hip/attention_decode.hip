@@ -25,7 +25,7 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
     int n_kv_head, int head_dim, int page_size, float scale, int window, const float* __restrict__ sinks,
-    float softcap) {
+    float softcap, const bf16_t* __restrict__ gate, long ldg) {
   __shared__ float q_s[AD_MAX_DPL * 64];
   __shared__ float p_s[AD_WAVES][64];
   __shared__ int page_s[AD_WAVES][64];
@@ -127,7 +127,8 @@ __global__ __launch_bounds__(256) void paged_attention_split_kernel(
       f[w] = (m_s[w] == -INFINITY) ? 0.f : __expf(m_s[w] - mx);
       lt += l_s[w] * f[w];
     }
-    const float inv = 1.0f / lt;
+    float inv = 1.0f / lt;
+    if (gate) inv *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));   // sigmoid gate of the head
 #pragma unroll
     for (int i = 0; i < AD_MAX_DPL; ++i) {
       const int d = lane + i * 64;
@@ -144,7 +145,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, hipStream_t stream) {
+    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
@@ -154,7 +155,7 @@ extern "C" int mgpt_paged_attention_split_bf16(
   hipLaunchKernelGGL(paged_attention_split_kernel, dim3(n_tokens, n_head), dim3(256), 0, stream,
                      (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,
                      block_tables, max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim,
-                     page_size, scale, window, sinks, softcap);
+                     page_size, scale, window, sinks, softcap, (const bf16_t*)gate, ldg);
   return mgpt_last_error();
 }
 
@@ -170,7 +171,8 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, const int* __restrict__ q_req, int n_tokens, int n_head,
-    int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks, float softcap) {
+    int n_kv_head, int page_size, float scale, int window, const float* __restrict__ sinks, float softcap,
+    const bf16_t* __restrict__ gate, long ldg) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   __shared__ float m_s[AD_WAVES], l_s[AD_WAVES];
@@ -290,7 +292,9 @@ __global__ __launch_bounds__(256) void paged_attention_split_fast_kernel(
       lt += l_s[w] * f;
       a += acc_s[w][tid] * f;
     }
-    out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(a / lt);
+    float res = a / lt;
+    if (gate) res *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));
+    out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(res);
   }
 }
 
@@ -298,7 +302,7 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, hipStream_t stream) {
+    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
@@ -309,7 +313,8 @@ extern "C" int mgpt_paged_attention_split_fast_bf16(
 #define AD_LAUNCH(DD)                                                                                   \
   hipLaunchKernelGGL(paged_attention_split_fast_kernel<DD>, grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,       \
-                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks, softcap)
+                     max_blocks, cu_q, seq_lens, q_req, n_tokens, n_head, n_kv_head, page_size, scale, window, sinks, softcap, \
+                     (const bf16_t*)gate, ldg)
   switch (head_dim) {
     case 16: AD_LAUNCH(16); break;
     case 32: AD_LAUNCH(32); break;

@@ -70,7 +70,7 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ positions,
     const int* __restrict__ q_req, const int* __restrict__ cu_q, int n_head, int n_kv_head, int page_shift,
     int num_pages, unsigned int page_bytes, float scale_log2e, int window, const float* __restrict__ sinks,
-    float cap_log2e) {
+    float cap_log2e, const bf16_t* __restrict__ gate, long ldg) {
   constexpr int LPK = D / 8;     // lanes per key
   constexpr int KPI = 64 / LPK;  // keys per load instruction
   constexpr int ROWS = AW_WAVES * KPI;      // partial results: one per (key subgroup, wave)
@@ -225,7 +225,9 @@ __global__ __launch_bounds__(AW_WAVES * 64) void paged_attention_decode_kernel(
       for (int w = 0; w < AW_WAVES; ++w) mx = fmaxf(mx, m_s[w]);
       lt += __builtin_amdgcn_exp2f(sink - mx);
     }
-    out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(a / lt);
+    float res = a / lt;
+    if (gate) res *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)n * ldg + h])));   // sigmoid gate of the head
+    out[(long)n * ldo + (long)h * D + tid] = float_to_bf16(res);
   }
 }
 
@@ -239,7 +241,7 @@ extern "C" int mgpt_paged_attention_decode_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int* cu_q,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale, int window,
-    int identity, const float* sinks, float softcap, hipStream_t stream) {
+    int identity, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !positions || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || page_size <= 0 ||
@@ -260,7 +262,8 @@ extern "C" int mgpt_paged_attention_decode_bf16(
   hipLaunchKernelGGL((paged_attention_decode_kernel<DD, ID>), grid, block, 0, stream, (const bf16_t*)q, ldq, \
                      (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool, block_tables,          \
                      max_blocks, positions, q_req, cu_q, n_head, n_kv_head, page_shift, num_pages, page_bytes, \
-                     scale_log2e, window, sinks, softcap > 0.f ? softcap * 1.4426950408889634f : 0.f)
+                     scale_log2e, window, sinks, softcap > 0.f ? softcap * 1.4426950408889634f : 0.f, \
+                     (const bf16_t*)gate, ldg)
 #define AW_LAUNCH(DD)              \
   do {                             \
     if (identity) AW_LAUNCH2(DD, true); \

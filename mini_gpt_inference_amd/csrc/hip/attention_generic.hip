@@ -9,7 +9,8 @@
 // attention: S = q k^T * scale; a query at absolute position p sees the keys at
 // positions max(0, p-window+1)..p of its own request (window 0 = all of them);
 // softmax over keys in 32-bit (with `sinks`, one more term exp(sinks[head]) in its denominator that
-// has no value; with `softcap` > 0 every score becomes softcap * tanh(score / softcap) first);
+// has no value; with `softcap` > 0 every score becomes softcap * tanh(score / softcap) first; with `gate`
+// a head's output is multiplied by sigmoid(gate[token][head]));
 // y = P v (reference: src/minigpt_infer/model.py:61-87,
 // the rule col <= cache_len + row of src/minigpt_infer/batch.py:202-227).
 //
@@ -72,7 +73,7 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
     const T* __restrict__ vpool, const int* __restrict__ block_tables, int max_blocks,
     const int* __restrict__ cu_q, const int* __restrict__ seq_lens, const int* __restrict__ q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* __restrict__ sinks, float softcap) {
+    const float* __restrict__ sinks, float softcap, const T* __restrict__ gate, long ldg) {
   __shared__ float q_s[MAX_DPL * MGPT_WAVE];
   __shared__ float p_s[MGPT_WAVE];
   __shared__ int page_s[MGPT_WAVE];
@@ -147,7 +148,11 @@ __global__ __launch_bounds__(64) void paged_attention_generic_kernel(
 #pragma unroll
     for (int i = 0; i < MAX_DPL; ++i) acc[i] *= alpha;
   }
-  const float inv_l = 1.0f / l;
+  float inv_l = 1.0f / l;
+  if (gate) {   // the head's output times sigmoid(gate[token][head])
+    const float gv = to_float<T>(gate[(long)n * ldg + h]);
+    inv_l *= 1.0f / (1.0f + (FAST_EXP ? __expf(-gv) : expf(-gv)));
+  }
 #pragma unroll
   for (int i = 0; i < MAX_DPL; ++i) {
     const int d = lane + i * MGPT_WAVE;
@@ -162,7 +167,7 @@ extern "C" int mgpt_paged_attention_generic(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int dtype, int fast_exp, const float* sinks, float softcap, hipStream_t stream) {
+    int dtype, int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
   if (n_tokens == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens || !q_req) return MGPT_ERR_NULL;
   if (n_tokens < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 || head_dim <= 0 ||
@@ -173,7 +178,8 @@ extern "C" int mgpt_paged_attention_generic(
 #define LAUNCH(T, F)                                                                              \
   hipLaunchKernelGGL((paged_attention_generic_kernel<T, F>), grid, block, 0, stream, (const T*)q, ldq, \
                      (T*)out, ldo, (const T*)kpool, (const T*)vpool, block_tables, max_blocks, cu_q,  \
-                     seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim, page_size, scale, window, sinks, softcap)
+                     seq_lens, q_req, n_tokens, n_head, n_kv_head, head_dim, page_size, scale, window, sinks, softcap, \
+                     (const T*)gate, ldg)
   if (dtype == MGPT_F32) {
     if (fast_exp) LAUNCH(float, true); else LAUNCH(float, false);
   } else if (dtype == MGPT_BF16) {

@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vpool,
     const int* __restrict__ block_tables, int max_blocks, const int* __restrict__ cu_q,
     const int* __restrict__ seq_lens, int n_head, int n_kv_head, int page_size, float scale, int window,
-    int single_below, const float* __restrict__ sinks, float softcap) {
+    int single_below, const float* __restrict__ sinks, float softcap, const bf16_t* __restrict__ gate, long ldg) {
   constexpr int THREADS = 256 * G;
   constexpr int SB = PF_KT * G;    // keys staged per step
   // Key and value rows in LDS: as long as the head size where that is a power of two, the 16-byte
@@ -335,7 +335,9 @@ __global__ __launch_bounds__(256 * G) void prefill_attention_kernel(
       for (int i = 0; i < 4; ++i) o[dt][i] *= a;
   }
   if (q_ok) {
-    const float inv = 1.0f / l;
+    float inv = 1.0f / l;
+    if (gate)   // the head's output times sigmoid(gate[token][head])
+      inv *= __builtin_amdgcn_rcpf(1.0f + __expf(-bf16_to_float(gate[(long)(q_start + my_q) * ldg + h])));
     bf16_t* orow = out + (long)(q_start + my_q) * ldo + (long)h * D;
     // a lane's four neighbouring channels of a tile are one 8-byte store (the launcher has checked
     // that rows start 8 bytes aligned)
@@ -358,7 +360,7 @@ extern "C" int mgpt_prefill_attention_bf16(
     const void* q, long ldq, void* out, long ldo, const void* kpool, const void* vpool,
     const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req,
     int max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    int single_below, const float* sinks, float softcap, hipStream_t stream) {
+    int single_below, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream) {
   if (n_req == 0 || max_q_len == 0) return MGPT_OK;
   if (!q || !out || !kpool || !vpool || !block_tables || !cu_q || !seq_lens) return MGPT_ERR_NULL;
   if (n_req < 0 || max_q_len < 0 || n_head <= 0 || n_kv_head <= 0 || (n_head % n_kv_head) != 0 ||
@@ -382,7 +384,7 @@ extern "C" int mgpt_prefill_attention_bf16(
     hipLaunchKernelGGL((prefill_attention_kernel<DD, GG>), grid, dim3(256 * GG), lds_bytes, stream,             \
                        (const bf16_t*)q, ldq, (bf16_t*)out, ldo, (const bf16_t*)kpool, (const bf16_t*)vpool,    \
                        block_tables, max_blocks, cu_q, seq_lens, n_head, n_kv_head, page_size, scale, window,   \
-                       single_below, sinks, softcap);                                                                          \
+                       single_below, sinks, softcap, (const bf16_t*)gate, ldg);                                                                          \
   }
   // Two wave groups halve the walk of a tile over its keys; one group leaves LDS for a second
   // workgroup on the compute unit.  The first serves a step with few tiles, the second one with many.

@@ -10,17 +10,17 @@ extern "C" {
 int mgpt_paged_attention_split_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int*
     q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, hipStream_t stream);
+    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
 // attention_decode.hip
 int mgpt_paged_attention_split_fast_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool,
     const void* vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const
     int* q_req, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window,
-    const float* sinks, float softcap, hipStream_t stream);
+    const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
 // attention_decode_wide.hip
 int mgpt_paged_attention_decode_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const
     void* vpool, const int* block_tables, int max_blocks, const int* positions, const int* q_req, const int*
     cu_q, int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, int num_pages, float scale,
-    int window, int identity, const float* sinks, float softcap, hipStream_t stream);
+    int window, int identity, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
 // attention_generic.hip
 int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, void* kpool, void* vpool, const
     int* slot_mapping, int n_tokens, int n_kv_head, int head_dim, int page_size, hipStream_t stream);
@@ -28,12 +28,12 @@ int mgpt_kv_write(const void* qkv, int dtype, long ld, int k_off, int v_off, voi
 int mgpt_paged_attention_generic(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, const int* q_req,
     int n_tokens, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int dtype,
-    int fast_exp, const float* sinks, float softcap, hipStream_t stream);
+    int fast_exp, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
 // attention_prefill.hip
 int mgpt_prefill_attention_bf16(const void* q, long ldq, void* out, long ldo, const void* kpool, const void*
     vpool, const int* block_tables, int max_blocks, const int* cu_q, const int* seq_lens, int n_req, int
     max_q_len, int n_head, int n_kv_head, int head_dim, int page_size, float scale, int window, int
-    single_below, const float* sinks, float softcap, hipStream_t stream);
+    single_below, const float* sinks, float softcap, const void* gate, long ldg, hipStream_t stream);
 // embed_norm.hip
 int mgpt_embed(const int* ids, const int* pos, const void* tok, const void* postab, float* x, int n_tokens,
     int width, int table_dtype, hipStream_t stream);
@@ -158,8 +158,6 @@ int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_off, int v_of
     int head_dim, int value_dim, int head_stride, const int* positions, const float* freq, int rot_dims, float norm_eps,
     const float* mix_lambda, void* v_other, long ld_other, int mix_mode, void* kpool, void* vpool,
     const int* slot_mapping, int page_size, int n_tokens, hipStream_t stream);
-int mgpt_head_gate(void* y, int dtype, long ldy, int head_stride, int width, const void* gate, int gate_dtype,
-    long ldg, int n_rows, int n_head, hipStream_t stream);
 // decay_state.hip
 int mgpt_decay_state(const void* z, int dtype, long ldz, int q_off, int k_off, int v_off, int g_off, int n_head,
     int head_dim, int value_dim, int act, const int* positions, const float* freq, int rot_dims, float k_scale,
@@ -219,6 +217,5 @@ int mgpt_linear_mfma_grouped(const void* act, long lda, const void* w, long w_st
   X(mgpt_rms_norm) \
   X(mgpt_rms_post_norm) \
   X(mgpt_qk_prepare) \
-  X(mgpt_head_gate) \
   X(mgpt_decay_state) \
   X(mgpt_decay_state_chunked)

@@ -107,30 +107,3 @@ extern "C" int mgpt_qk_prepare(void* z, int dtype, long ldz, int q_off, int k_of
                      v_other, ld_other, mix_mode, kpool, vpool, slot_mapping, page_size, n_tokens);
   return mgpt_last_error();
 }
-
-// y[n, h, 0 .. width) *= sigmoid(gate[n, h]): one number per head in front of the output projection
-__global__ __launch_bounds__(256) void head_gate_kernel(void* __restrict__ y, int dtype, long ldy, int head_stride, int width,
-                                                        const void* __restrict__ gate, int gate_dtype, long ldg,
-                                                        int n_rows, int n_head) {
-  const long i = (long)blockIdx.x * 256 + threadIdx.x;
-  const long per_row = (long)n_head * width;
-  if (i >= (long)n_rows * per_row) return;
-  const int n = (int)(i / per_row);
-  const int rem = (int)(i - (long)n * per_row);
-  const int h = rem / width, c = rem - h * width;
-  const float g = load_f(gate, gate_dtype, (long)n * ldg + h);
-  const long at = (long)n * ldy + (long)h * head_stride + c;
-  store_f(y, dtype, at, load_f(y, dtype, at) / (1.0f + expf(-g)));
-}
-
-extern "C" int mgpt_head_gate(void* y, int dtype, long ldy, int head_stride, int width, const void* gate, int gate_dtype,
-                              long ldg, int n_rows, int n_head, hipStream_t stream) {
-  if (n_rows == 0) return MGPT_OK;
-  if (!y || !gate) return MGPT_ERR_NULL;
-  if (!dtype_ok(dtype) || !dtype_ok(gate_dtype)) return MGPT_ERR_BAD_DTYPE;
-  if (n_rows < 0 || n_head <= 0 || width <= 0 || head_stride < width) return MGPT_ERR_BAD_SHAPE;
-  const long total = (long)n_rows * n_head * width;
-  hipLaunchKernelGGL(head_gate_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, y, dtype, ldy,
-                     head_stride, width, gate, gate_dtype, ldg, n_rows, n_head);
-  return mgpt_last_error();
-}

@@ -8,7 +8,7 @@ from . import kernels
 
 
 def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int, sinks=None,
-                softcap: float = 0.0) -> bool:
+                softcap: float = 0.0, gate=None) -> bool:
     """A step with prompt portions.  The requests that lead the step with one token each (a scheduler
     puts the decoding requests first) go to the decode kernel, token n being request n; the rest,
     prompt portions mostly, to the MFMA tile kernel, which would spend a 64-query tile on a single
@@ -21,19 +21,19 @@ def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, w
     rest = ctx.n_req - lead
     if lead and rest and kernels.prefill_attention_bf16(
             q, out, k_pool, v_pool, group.block_tables[lead:], ctx.cu_q[lead:], ctx.seq_lens[lead:], rest,
-            ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap):
+            ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate):
         if kernels.paged_attention_decode_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req,
-                                               lead, n_head, scale, window, identity=True, sinks=sinks, softcap=softcap):
+                                               lead, n_head, scale, window, identity=True, sinks=sinks, softcap=softcap, gate=gate):
             return True
         # the decode kernel refuses this head or page size: the tile kernel for the leading requests too
         return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap)
+                                              lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                          ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap)
+                                          ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate)
 
 
 def _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int, sinks=None,
-                       softcap: float = 0.0) -> bool:
+                       softcap: float = 0.0, gate=None) -> bool:
     """A step with prompt portions that is padded to its bucket's sizes (a graph replays it for every
     step of the bucket): which request brings how many tokens is known on the device only.  The
     decode kernel goes over the step's first `ctx.lead_cap` tokens (decoding requests lead a step)
@@ -44,16 +44,18 @@ def _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: f
     lead = min(ctx.lead_cap, ctx.n_rows)
     singles = lead > 0 and kernels.paged_attention_decode_bf16(
         q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, lead, n_head, scale, window,
-        cu_q=ctx.cu_q, sinks=sinks, softcap=softcap)
+        cu_q=ctx.cu_q, sinks=sinks, softcap=softcap, gate=gate)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens, r,
                                           ctx.n_rows, n_head, scale, window, single_below=lead if singles else 0,
-                                          sinks=sinks, softcap=softcap)
+                                          sinks=sinks, softcap=softcap, gate=gate)
 
 
 def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
-                    group, n_head: int, scale: float, window: int, sinks=None, softcap: float = 0.0) -> None:
+                    group, n_head: int, scale: float, window: int, sinks=None, softcap: float = 0.0,
+                    gate=None) -> None:
     """Attention of the step's tokens (rows of q) over their requests' pages.  softcap > 0: scores
-    pass cap * tanh(score / cap) before the softmax.
+    pass cap * tanh(score / cap) before the softmax.  gate ([tokens, >= heads], the queries' dtype): a head's
+    output is multiplied by sigmoid(gate[token][head]).
 
     On the bfloat16 path a decode-only step (token n is request n's one token) uses the kernel
     laid out for a decode step's latency, steps with prompt portions the MFMA tile kernel and the
@@ -63,17 +65,17 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
     if q.dtype == torch.bfloat16 and not ctx.exact:
         if ctx.decode_only and kernels.paged_attention_decode_bf16(
                 q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req, n, n_head, scale, window,
-                identity=True, sinks=sinks, softcap=softcap):
+                identity=True, sinks=sinks, softcap=softcap, gate=gate):
             return
         if not ctx.decode_only and not ctx.padded and _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head, scale,
-                                                                  window, sinks, softcap):
+                                                                  window, sinks, softcap, gate):
             return
         if not ctx.decode_only and ctx.padded and _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head,
-                                                                     scale, window, sinks, softcap):
+                                                                     scale, window, sinks, softcap, gate):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                              ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap):
+                                              ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate):
             return
     kernels.paged_attention_generic(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                     ctx.q_req, n, r, n_head, scale, window, fast_exp=not ctx.exact, sinks=sinks,
-                                    softcap=softcap)
+                                    softcap=softcap, gate=gate)

@@ -178,6 +178,17 @@ def kv_write(qkv: torch.Tensor, k_off: int, v_off: int, k_pool: torch.Tensor, v_
     _check(rc, "kv_write")
 
 
+def _gate_args(gate: Optional[torch.Tensor], q: torch.Tensor, n_tokens: int, n_head: int):
+    """(pointer, row stride) of the optional gate [tokens, >= heads] in q's dtype: a head's attention output is
+    multiplied by sigmoid(gate[token][head])."""
+    if gate is None:
+        return None, 0
+    _need_cuda(gate)
+    _need(gate.dtype == q.dtype and gate.dim() == 2 and gate.stride(1) == 1 and gate.shape[0] >= n_tokens
+          and gate.shape[1] >= n_head, "the heads' gate must be rows [tokens, >= heads] in the queries' dtype")
+    return _ptr(gate), gate.stride(0)
+
+
 def _check_attention_args(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req, n_tokens, n_req, n_head):
     _need_cuda(q, out, k_pool, v_pool, block_tables, cu_q, seq_lens, q_req)
     _need(k_pool.shape == v_pool.shape and k_pool.dim() == 4 and k_pool.is_contiguous() and v_pool.is_contiguous(),
@@ -201,7 +212,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
                             block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                             q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
                             window: int = 0, fast_exp: bool = False, sinks: Optional[torch.Tensor] = None,
-                            softcap: float = 0.0) -> None:
+                            softcap: float = 0.0, gate: Optional[torch.Tensor] = None) -> None:
     """Causal attention of the step's tokens over their requests' pages (any q_len, any dtype).
     sinks: float32 [n_head], one more term exp(sinks[h]) in every softmax denominator of head h.
     softcap > 0: every score becomes softcap * tanh(score / softcap) before the softmax."""
@@ -212,7 +223,7 @@ def paged_attention_generic(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Te
     rc = library.kernels().mgpt_paged_attention_generic(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), float(softcap), _stream())
+        page_size, float(scale), int(window), _dtype_code(q), int(fast_exp), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head), _stream())
     _check(rc, "paged_attention_generic")
 
 
@@ -487,7 +498,7 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
                                block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor,
                                q_req: torch.Tensor, n_tokens: int, n_req: int, n_head: int, scale: float,
                                window: int = 0, fast: bool = True, sinks: Optional[torch.Tensor] = None,
-                               softcap: float = 0.0) -> bool:
+                               softcap: float = 0.0, gate: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention with each (token, head)'s keys split over four waves.  False if refused.
     fast=False keeps to the variant that takes every head size."""
     if q.dtype != torch.bfloat16:
@@ -503,7 +514,7 @@ def paged_attention_split_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch
     rc = fn(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), _ptr(q_req), n_tokens, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), _ptr(sinks), float(softcap), _stream())
+        page_size, float(scale), int(window), _ptr(sinks), float(softcap), *_gate_args(gate, q, n_tokens, n_head), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_split_bf16")
@@ -514,7 +525,8 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
                                 block_tables: torch.Tensor, positions: torch.Tensor, q_req: torch.Tensor,
                                 n_tokens: int, n_head: int, scale: float, window: int = 0,
                                 identity: bool = False, cu_q: Optional[torch.Tensor] = None,
-                                sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> bool:
+                                sinks: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                                gate: Optional[torch.Tensor] = None) -> bool:
     """bfloat16 attention for single tokens (one query per request and step), keys split over eight
     waves.  positions[n] is token n's absolute position, q_req[n] its block table row or -1 for a
     padded token; identity=True promises q_req[n] in (n, -1).  With cu_q (the requests' token offsets;
@@ -549,7 +561,8 @@ def paged_attention_decode_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torc
     rc = library.kernels().mgpt_paged_attention_decode_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(positions), _ptr(q_req), _ptr(cu_q), n_tokens, n_head, n_kv_head, head_dim, page_size,
-        num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), float(softcap), _stream())
+        num_pages, float(scale), int(window), 1 if identity else 0, _ptr(sinks), float(softcap),
+        *_gate_args(gate, q, n_tokens, n_head), _stream())
     if rc == -2:
         return False
     _check(rc, "paged_attention_decode_bf16")
@@ -659,7 +672,8 @@ def linear_mfma(a: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
 def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                            block_tables: torch.Tensor, cu_q: torch.Tensor, seq_lens: torch.Tensor, n_req: int,
                            max_q_len: int, n_head: int, scale: float, window: int = 0,
-                           single_below: int = 0, sinks: Optional[torch.Tensor] = None, softcap: float = 0.0) -> bool:
+                           single_below: int = 0, sinks: Optional[torch.Tensor] = None, softcap: float = 0.0,
+                           gate: Optional[torch.Tensor] = None) -> bool:
     """MFMA tile attention for steps with prompt portions (every request's tokens are consecutive
     rows of q from cu_q; a request may bring none).  Requests that bring exactly one token, and that
     among the step's first `single_below` tokens, are left to another kernel.  False when it does
@@ -686,7 +700,8 @@ def prefill_attention_bf16(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Ten
     rc = library.kernels().mgpt_prefill_attention_bf16(
         _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_pool), _ptr(v_pool), _ptr(block_tables),
         block_tables.shape[1], _ptr(cu_q), _ptr(seq_lens), n_req, max_q_len, n_head, n_kv_head, head_dim,
-        page_size, float(scale), int(window), int(single_below), _ptr(sinks), float(softcap), _stream())
+        page_size, float(scale), int(window), int(single_below), _ptr(sinks), float(softcap),
+        *_gate_args(gate, q, q.shape[0], n_head), _stream())
     if rc == -2:
         return False
     _check(rc, "prefill_attention_bf16")
@@ -1352,17 +1367,6 @@ def qk_prepare(z: torch.Tensor, q_off: int, k_off: int, v_off: int, n_head: int,
         _ptr(v_other), v_other.stride(0) if v_other is not None else 0, int(mix_mode), _ptr(k_pool), _ptr(v_pool),
         _ptr(slot_mapping), page_size, n_tokens, _stream())
     _check(rc, "qk_prepare")
-
-
-def head_gate(y: torch.Tensor, gate: torch.Tensor, n_rows: int, n_head: int, width: int, head_stride: int) -> None:
-    """y[n, h * head_stride + c] *= sigmoid(gate[n, h]) for c < width."""
-    _need_cuda(y, gate)
-    _rows_2d("head_gate y", y, n_rows)
-    _rows_2d("head_gate gate", gate, n_rows)
-    _need(y.shape[1] >= (n_head - 1) * head_stride + width and gate.shape[1] >= n_head, "head_gate: rows too narrow")
-    rc = library.kernels().mgpt_head_gate(_ptr(y), _dtype_code(y), y.stride(0), head_stride, width, _ptr(gate),
-                                          _dtype_code(gate), gate.stride(0), n_rows, n_head, _stream())
-    _check(rc, "head_gate")
 
 
 def decay_state(z: torch.Tensor, q_off: int, k_off: int, v_off: int, g_off: int, n_head: int, head_dim: int,

@@ -39,7 +39,7 @@ def kernels() -> ctypes.CDLL:
         lib.mgpt_layernorm.argtypes = [P, P, P, P, P, I, I, F, I, P]
         lib.mgpt_linear_generic.argtypes = [P, I, L, P, I, P, P, I, L, I, I, I, I, P]
         lib.mgpt_kv_write.argtypes = [P, I, L, I, I, P, P, P, I, I, I, I, P]
-        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, F, P]
+        lib.mgpt_paged_attention_generic.argtypes = [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, P, F, P, L, P]
         lib.mgpt_sample.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P, P, P, I, P]
         lib.mgpt_sample_advance.argtypes = [P, L, I, I, I, P, P, P, P, P, c_ulonglong, P,
                                             P, P, P, P, P, P, P, I, I, I, I, P, P, I, I, P, P, I, P]
@@ -127,15 +127,15 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_linear_skinny_partials": [I, I, I, I, I],
         "mgpt_linear_skinny_row_groups": [I, I, I],
         "mgpt_fold_layernorm": [P, P, P, P, P, P, P, I, I, P],
-        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P],
-        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P],
-        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P],
+        "mgpt_paged_attention_split_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, P],
+        "mgpt_paged_attention_split_fast_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, P, F, P, L, P],
+        "mgpt_paged_attention_decode_bf16": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, P],
         "mgpt_linear_mfma": [P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_shape": [I, I, P, L, P, P, P, I, L, I, I, I, I, P, L, P],
         "mgpt_linear_mfma_partials": [I, I, I, I],
         "mgpt_linear_mfma_parts": [P, L, P, P, P, L, I, I, I, P],
         "mgpt_linear_mfma_qkv": [P, L, P, P, P, L, I, I, I, P, P, P, I, I, I, I, I, I, P],
-        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, F, P],
+        "mgpt_prefill_attention_bf16": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, I, F, I, I, P, F, P, L, P],
         # a residual that is still a sum: base, partials, n_parts, part_stride, token table, position table, ids, positions
         "mgpt_fused_attention_decode": [P, P, I, L, P, P, P, P, P, P, P, P, F, P, P, P, P, P, L, P, P, P, P, I, P, P,
                                         I, I, I, I, I, I, F, P],
@@ -163,7 +163,6 @@ def _declare_optional(lib: ctypes.CDLL) -> None:
         "mgpt_rms_norm": [P, I, L, P, P, F, F, F, P, I, L, I, P, I, L, I, P, L, I, I, I, I, I, I, P],
         "mgpt_rms_post_norm": [P, P, P, P, P, P, P, P, I, F, P, P, F, F, F, P, P, I, I, I, P],
         "mgpt_qk_prepare": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, L, I, P, P, P, I, I, P],
-        "mgpt_head_gate": [P, I, L, I, I, P, I, L, I, I, P],
         "mgpt_decay_state": [P, I, L, I, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, F, P, I, L, P],
         "mgpt_decay_state_chunked": [P, I, L, I, I, I, I, I, I, I, P, P, I, F, P, P, P, P, I, I, P, P, L, P],
         "mgpt_expert_route": [P, P, P, I, I, I, P, P, P, P, I, I, I, P],

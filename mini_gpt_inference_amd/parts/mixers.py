@@ -374,9 +374,9 @@ class GatedAttention(Mixer):
                            norm_eps=self.qk_norm_eps, mix_lambda=self.mix if mode == 2 else None, v_other=other,
                            mix_mode=mode, k_pool=k_pool, v_pool=v_pool, slot_mapping=group.slot_mapping)
         y = ws.get("attn_out", n, self.n_head * s, ctx.dtype)
-        attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, 0, softcap=self.softcap)
-        if self.has_gate:
-            kernels.head_gate(y, z[:, self.g_off:], n, self.n_head, s, s)
+        # (the gate per head is applied by the attention kernel as it stores a head's output)
+        attention_ops.paged_attention(ctx, z, y, k_pool, v_pool, group, self.n_head, self.scale, 0, softcap=self.softcap,
+                                      gate=z[:, self.g_off:] if self.has_gate else None)
         linear_add(ctx, y, self.out_padded, None, x, n)
 
 

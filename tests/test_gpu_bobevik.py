@@ -1,6 +1,6 @@
 """Bobevik on the GPU against the plain implementation (tests/plain_bobevik.py): each new kernel
 alone (RMS norms, the step between two sublayers, rotation / head norm / value mixing / page store,
-the gate per head, the decaying state, capped scores, the gated unit's activations); whole prompts
+the decaying state, capped scores and the gate per head in the attention kernels, the gated unit's activations); whole prompts
 against token-by-token decoding, portions down to two tokens and mixed batches with pages, request
 slots and states used again, steps that want no logits, in 32-bit and bfloat16; long decoding;
 configurations drawn at random; greedy generation through LLMEngine."""
@@ -195,28 +195,18 @@ def test_the_plain_rotation_agrees_with_its_one_position_form():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_gate_per_head(dtype):
-    g = torch.Generator().manual_seed(3)
-    n, H, E, stride = 5, 3, 20, 32
-    y = _rnd(g, n, H * stride, dtype=dtype)
-    gate = _rnd(g, n, H + 2, dtype=dtype, scale=2.0)
-    yd = y.to(DEV)
-    kernels.head_gate(yd, gate.to(DEV), n, H, E, stride)
-    want = _d(y).view(n, H, stride).clone()
-    want[:, :, :E] *= P.sigmoid(_d(gate[:, :H]))[:, :, None]
-    helpers.assert_close(yd, want.reshape(n, -1), dtype, "head gate")
-    assert torch.equal(yd.view(n, H, stride)[:, :, E:].cpu(), y.view(n, H, stride)[:, :, E:])
-
-
-@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("kind,f", [("silu", P.silu), ("relu", lambda z: torch.clamp(z, min=0.0)),
                                     ("gelu_tanh", lambda z: 0.5 * z * (1 + torch.tanh(0.7978845608028654 * (z + 0.044715 * z ** 3))))])
 def test_gated_unit_activations(dtype, kind, f):
     g = torch.Generator().manual_seed(4)
-    z = _rnd(g, 7, 2 * 36, dtype=dtype, scale=2.0)
-    act = torch.zeros(7, 36, dtype=TDT[dtype], device=DEV)
-    kernels.gated_unit(z.to(DEV), act, 7, 36, fast=dtype == "bfloat16", activation=kind)
-    helpers.assert_close(act, f(_d(z[:, :36])) * _d(z[:, 36:]), dtype, kind)
+    for hidden in (36, 40, 320):          # (multiples of 8 take the kernel with 16-byte loads in bfloat16)
+        z = _rnd(g, 7, 2 * hidden, dtype=dtype, scale=2.0)
+        for fast in (False, True):
+            act = torch.full((8, hidden), 3.0, dtype=TDT[dtype], device=DEV)
+            kernels.gated_unit(z.to(DEV), act, 7, hidden, fast=fast, activation=kind)
+            helpers.assert_close(act[:7], f(_d(z[:, :hidden])) * _d(z[:, hidden:]), dtype if not fast else "bfloat16",
+                                 f"{kind} {hidden}")
+            assert (act[7] == 3.0).all()
 
 
 def _state_case(g, dtype, lens, H, D, E):
@@ -404,6 +394,8 @@ def test_capped_scores_in_attention_with_a_key_that_stands_out(dtype):
     want = P.causal_softmax_attention(_d(q), _d(k), _d(v), scale, cap)
     uncapped = P.causal_softmax_attention(_d(q), _d(k), _d(v), scale, None)
     assert float((want[-1] - uncapped[-1]).abs().max()) > 0.3
+    gate = _rnd(g, T, H + 3, dtype=dtype, scale=2.0)        # one number a token and head, behind a sigmoid
+    gated = want * P.sigmoid(_d(gate[:, :H]))[:, :, None]
     pages = T // page
     perm = torch.randperm(pages, generator=g)
     kp = torch.zeros(pages, G, page, D, dtype=TDT[dtype])
@@ -418,6 +410,10 @@ def test_capped_scores_in_attention_with_a_key_that_stands_out(dtype):
                                     perm.to(torch.int32).view(1, pages).to(DEV), i32([0, T - first]), i32([T]),
                                     i32([0] * (T - first)), T - first, 1, H, scale, softcap=cap)
     helpers.assert_close(out[:T - first], want[first:].reshape(T - first, H * D), dtype, "capped attention")
+    kernels.paged_attention_generic(q[first:].reshape(T - first, H * D).to(DEV), out, kp.to(DEV), vp.to(DEV),
+                                    perm.to(torch.int32).view(1, pages).to(DEV), i32([0, T - first]), i32([T]),
+                                    i32([0] * (T - first)), T - first, 1, H, scale, softcap=cap, gate=gate[first:].to(DEV))
+    helpers.assert_close(out[:T - first], gated[first:].reshape(T - first, H * D), dtype, "capped and gated attention")
 
 
 @pytest.mark.parametrize("D", [32, 64, 128])
@@ -444,21 +440,25 @@ def test_capped_scores_in_the_bfloat16_attention_kernels(D):
     first = 100
     n = T - first
     qd = q[first:].reshape(n, H * D).to(DEV)
-    out = torch.zeros(n, H * D, dtype=torch.bfloat16, device=DEV)
-    assert kernels.prefill_attention_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), 1, n, H, scale, softcap=cap)
-    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "tile kernel")
-    out.zero_()
-    assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
-                                              softcap=cap)
-    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "split kernel")
-    out.zero_()
-    assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
-                                              fast=False, softcap=cap)
-    helpers.assert_close(out, want[first:].reshape(n, H * D), "bfloat16", "split kernel, general variant")
-    one = torch.zeros(1, H * D, dtype=torch.bfloat16, device=DEV)
-    assert kernels.paged_attention_decode_bf16(qd[n - 1:], one, kp, vp, bt, i32([T - 1]), i32([0]), 1, H, scale,
-                                               identity=True, softcap=cap)
-    helpers.assert_close(one, want[T - 1:].reshape(1, H * D), "bfloat16", "decode kernel")
+    gate = _rnd(g, n, H + 5, dtype="bfloat16", scale=2.0)
+    for gd in (None, gate.to(DEV)):
+        ref = want[first:] if gd is None else want[first:] * P.sigmoid(_d(gate[:, :H]))[:, :, None]
+        ref = ref.reshape(n, H * D)
+        out = torch.zeros(n, H * D, dtype=torch.bfloat16, device=DEV)
+        assert kernels.prefill_attention_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), 1, n, H, scale, softcap=cap, gate=gd)
+        helpers.assert_close(out, ref, "bfloat16", "tile kernel")
+        out.zero_()
+        assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
+                                                  softcap=cap, gate=gd)
+        helpers.assert_close(out, ref, "bfloat16", "split kernel")
+        out.zero_()
+        assert kernels.paged_attention_split_bf16(qd, out, kp, vp, bt, i32([0, n]), i32([T]), i32([0] * n), n, 1, H, scale,
+                                                  fast=False, softcap=cap, gate=gd)
+        helpers.assert_close(out, ref, "bfloat16", "split kernel, general variant")
+        one = torch.zeros(1, H * D, dtype=torch.bfloat16, device=DEV)
+        assert kernels.paged_attention_decode_bf16(qd[n - 1:], one, kp, vp, bt, i32([T - 1]), i32([0]), 1, H, scale,
+                                                   identity=True, softcap=cap, gate=None if gd is None else gd[n - 1:])
+        helpers.assert_close(one, ref[n - 1:], "bfloat16", "decode kernel")
 
 
 # ---------------------------------------------------------------- the model through the step function
