@@ -23,13 +23,15 @@ def _mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, w
             q, out, k_pool, v_pool, group.block_tables[lead:], ctx.cu_q[lead:], ctx.seq_lens[lead:], rest,
             ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate):
         if kernels.paged_attention_decode_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.positions, ctx.q_req,
-                                               lead, n_head, scale, window, identity=True, sinks=sinks, softcap=softcap, gate=gate):
+                                               lead, n_head, scale, window, identity=True, sinks=sinks,
+                                               softcap=softcap, gate=gate):
             return True
         # the decode kernel refuses this head or page size: the tile kernel for the leading requests too
         return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                               lead, 1, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate)
     return kernels.prefill_attention_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                          ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate)
+                                          ctx.n_req, ctx.max_q_len, n_head, scale, window, sinks=sinks, softcap=softcap,
+                                          gate=gate)
 
 
 def _padded_mixed_step(ctx, q, out, k_pool, v_pool, group, n_head: int, scale: float, window: int, sinks=None,
@@ -74,7 +76,8 @@ def paged_attention(ctx, q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tenso
                                                                      scale, window, sinks, softcap, gate):
             return
         if kernels.paged_attention_split_bf16(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
-                                              ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap, gate=gate):
+                                              ctx.q_req, n, r, n_head, scale, window, sinks=sinks, softcap=softcap,
+                                              gate=gate):
             return
     kernels.paged_attention_generic(q, out, k_pool, v_pool, group.block_tables, ctx.cu_q, ctx.seq_lens,
                                     ctx.q_req, n, r, n_head, scale, window, fast_exp=not ctx.exact, sinks=sinks,
